@@ -1,0 +1,121 @@
+// C ABI of libkfold_hip.so (declared in include/kfold_hip.h): argument checking, workspace
+// carving and kernel sequencing.  No torch types, no allocation, no synchronisation.
+#include "../../include/kfold_hip.h"
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "kernels.hpp"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+// Report a launch failure of the kernels enqueued since the last check.
+int check_launch(const char* what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(KFH_EHIP, "%s: %s", what, hipGetErrorString(e));
+    return KFH_OK;
+}
+
+inline size_t align_up(size_t x, size_t a = 256) { return (x + a - 1) / a * a; }
+inline bool dtype_ok(int t) { return t == KFH_BF16 || t == KFH_F32; }
+
+}  // namespace
+
+using namespace kfh;
+
+extern "C" {
+
+int kfh_version(void) { return 1; }
+const char* kfh_last_error(void) { return g_err; }
+
+// ------------------------------------------------------------------------------------------
+// triangle multiplication
+// ------------------------------------------------------------------------------------------
+size_t kfh_trimul_packed_bytes(int C) { return C == kC ? align_up(kTmBlobBytes) : 0; }
+
+int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w,
+                    const void* g_in_w, const void* ln_out_w, const void* ln_out_b,
+                    const void* p_out_w, const void* g_out_w, int w_dtype, int C, void* blob,
+                    void* stream_) {
+    if (C != kC) return fail(KFH_EUNSUPPORTED, "trimul_pack: C=%d, only C=128 is built", C);
+    if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "trimul_pack: bad w_dtype %d", w_dtype);
+    if (!p_in_w || !g_in_w || !p_out_w || !g_out_w || !blob)
+        return fail(KFH_EINVAL, "trimul_pack: null weight or blob pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* b = static_cast<char*>(blob);
+    // input phase: step cb = { p_in rows 32cb.., g_in rows 32cb.. }
+    for (int cb = 0; cb < 8; ++cb) {
+        launch_pack_blocks(p_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                           b + kTmInOff + (2 * cb) * kBlockBytes, stream);
+        launch_pack_blocks(g_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                           b + kTmInOff + (2 * cb + 1) * kBlockBytes, stream);
+    }
+    launch_pack_blocks(g_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE2, K_NATURAL, 1.f,
+                       b + kTmGateOff, stream);
+    launch_pack_blocks(p_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE4, K_HALF, 1.f, b + kTmOutOff,
+                       stream);
+    float* ln = reinterpret_cast<float*>(b + kTmLnOff);
+    launch_copy_f32(ln_in_w, w_dtype, ln, C, 1.f, stream);
+    launch_copy_f32(ln_in_b, w_dtype, ln + C, C, 0.f, stream);
+    launch_copy_f32(ln_out_w, w_dtype, ln + 2 * C, C, 1.f, stream);
+    launch_copy_f32(ln_out_b, w_dtype, ln + 3 * C, C, 0.f, stream);
+    return check_launch("trimul_pack");
+}
+
+size_t kfh_trimul_workspace_bytes(int N, int C) {
+    if (C != kC || N <= 0) return 0;
+    const size_t np = trimul_np(N);
+    const size_t planes_ab = align_up(2 * (size_t)C * np * np * 2);
+    const size_t planes_y = align_up((size_t)C * np * np * 2);
+    const size_t gate = align_up((size_t)N * N * C * 2);
+    return planes_ab + planes_y + gate;
+}
+
+int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, const void* residual,
+                       void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
+                       int direction, float eps, int io_dtype, void* stream_) {
+    if (C != kC) return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d, only C=128 is built", C);
+    if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "trimul_forward: bad shape B=%d N=%d", B, N);
+    if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "trimul_forward: bad io_dtype %d", io_dtype);
+    if (direction != KFH_OUTGOING && direction != KFH_INCOMING)
+        return fail(KFH_EINVAL, "trimul_forward: bad direction %d", direction);
+    if (!z || !mask || !blob || !out || !workspace)
+        return fail(KFH_EINVAL, "trimul_forward: null pointer argument");
+    if (out == z && residual != z)
+        return fail(KFH_EINVAL, "trimul_forward: out may alias z only when residual == z");
+    const size_t need = kfh_trimul_workspace_bytes(N, C);
+    if (workspace_bytes < need)
+        return fail(KFH_EINVAL, "trimul_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const int np = trimul_np(N);
+    const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
+    char* ws = static_cast<char*>(workspace);
+    uint16_t* planes_ab = reinterpret_cast<uint16_t*>(ws);
+    uint16_t* planes_y = reinterpret_cast<uint16_t*>(ws + align_up(2 * (size_t)C * np * np * 2));
+    uint16_t* gate = reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(planes_y) +
+                                                 align_up((size_t)C * np * np * 2));
+    const char* bl = static_cast<const char*>(blob);
+    for (int b = 0; b < B; ++b) {
+        const size_t off = (size_t)b * N * N * C * esz;
+        const char* zb = static_cast<const char*>(z) + off;
+        const char* rb = residual ? static_cast<const char*>(residual) + off : nullptr;
+        char* ob = static_cast<char*>(out) + off;
+        launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, gate, N, np,
+                         direction == KFH_INCOMING, eps, stream);
+        launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream);
+        launch_trimul_out(planes_y, gate, bl, rb, ob, io_dtype, N, np, eps, stream);
+    }
+    return check_launch("trimul_forward");
+}
+
+}  // extern "C"

@@ -1,0 +1,146 @@
+// Shared device helpers for the gfx950 (CDNA4) kernels of the Pairformer pair-update path.
+//
+// Conventions used by every kernel in this directory
+// --------------------------------------------------
+// * Wavefront = 64 lanes.  lane = threadIdx.x & 63, half = lane >> 5, col = lane & 31.
+// * MFMA v_mfma_f32_32x32x16_bf16, D[32x32] += A[32x16] * B[16x32]:
+//     A operand: lane holds A[row = col][k = 8*half + 0..7]          (8 bf16 = one "fragment")
+//     B operand: lane holds B[k = 8*half + 0..7][column = col]
+//     D / C    : lane holds D[row = 8*(v/4) + 4*half + (v%4)][column = col], v = 0..15
+//   A and B fragments have the same register shape, so one fragment of a
+//   [32 rows x 16 k] operand block can be fed to either side.
+// * "Fragment order" in memory: a [32 x 16] operand block is stored as 64 lanes x 16 bytes
+//   (1 KiB, lane-major), so that a wavefront loads or stores a whole fragment with one
+//   fully coalesced 16-byte-per-lane access.
+// * Because a contraction is a sum, the k-slots of a fragment may hold any permutation of
+//   the true k indices as long as both operands use the same one.  Accumulator registers
+//   converted to bf16 are re-used directly as fragments of the next MFMA: register group
+//   v = 8*ks + e (e = 0..7) becomes k-step ks, and lane (col, half) then holds the true
+//   indices  8*(e/4) + 4*half + (e%4) + 16*ks  (KPERM_ACC below).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/kfold_hip.h"   // KFH_BF16 / KFH_F32 and the error codes
+
+namespace kfh {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// round-to-nearest-even pack of two floats into one dword of two bf16 (lo = a, hi = b)
+__device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
+    bf16x2 v = {(__bf16)a, (__bf16)b};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ float sigmoidf_fast(float x) {
+    return fast_rcp(1.0f + fast_exp2(-kLog2e * x));
+}
+
+// Exchange between lane l and lane l^32.  r0/r1 hold {own, partner} in the lower half and
+// {partner, own} in the upper half, so symmetric reductions need no select.
+__device__ __forceinline__ float xhalf_max(float x) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xhalf_sum(float x) {
+    auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
+// 16 accumulator values -> two fragments (k-steps) in KPERM_ACC order.
+__device__ __forceinline__ void acc_to_frags(const f32x16& c, bf16x8& f0, bf16x8& f1) {
+    u32x4 a, b;
+    a[0] = pack_bf16(c[0], c[1]);   a[1] = pack_bf16(c[2], c[3]);
+    a[2] = pack_bf16(c[4], c[5]);   a[3] = pack_bf16(c[6], c[7]);
+    b[0] = pack_bf16(c[8], c[9]);   b[1] = pack_bf16(c[10], c[11]);
+    b[2] = pack_bf16(c[12], c[13]); b[3] = pack_bf16(c[14], c[15]);
+    f0 = __builtin_bit_cast(bf16x8, a);
+    f1 = __builtin_bit_cast(bf16x8, b);
+}
+
+// row index inside a 32x32 accumulator block for register v of this lane
+__device__ __forceinline__ int acc_row(int v, int half) { return 8 * (v >> 2) + 4 * half + (v & 3); }
+
+// ---------------------------------------------------------------------------------------
+// Staging tile of LayerNorm-ed rows in LDS: 128 bf16 channels per row, row stride 272 bytes
+// (16 bytes of padding keep 16-byte fragment reads of consecutive rows on distinct banks).
+// ---------------------------------------------------------------------------------------
+constexpr int kC = 128;            // channels of the pair representation handled by the fused kernels
+constexpr int kXS = 272;           // bytes per staged row
+constexpr int kKS = kC / 16;       // k-steps per 128-channel contraction
+
+// fragment ks (0..7) of staged row `row` for this lane: channels 16*ks + 8*half + 0..7
+__device__ __forceinline__ bf16x8 lds_frag(const char* tile, int row, int ks, int half) {
+    return *reinterpret_cast<const bf16x8*>(tile + row * kXS + ks * 32 + half * 16);
+}
+
+template <int IO> struct IoT;
+template <> struct IoT<KFH_BF16> { using type = uint16_t; };
+template <> struct IoT<KFH_F32> { using type = float; };
+
+// Load 8 consecutive channels of one row as floats.
+template <int IO>
+__device__ __forceinline__ void load8(const void* base, size_t elem_off, float (&x)[8]) {
+    if constexpr (IO == KFH_BF16) {
+        u32x4 w = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(base) + elem_off);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { x[2 * i] = bf16_lo(w[i]); x[2 * i + 1] = bf16_hi(w[i]); }
+    } else {
+        const f32x4* p = reinterpret_cast<const f32x4*>(static_cast<const float*>(base) + elem_off);
+        f32x4 a = p[0], b = p[1];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) { x[i] = a[i]; x[4 + i] = b[i]; }
+    }
+}
+
+// sum over the 16 lanes that share one row (lanes 16*g .. 16*g+15)
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __shfl_xor(v, 1);
+    v += __shfl_xor(v, 2);
+    v += __shfl_xor(v, 4);
+    v += __shfl_xor(v, 8);
+    return v;
+}
+
+// LayerNorm of one 128-channel row held as 8 channels per lane over 16 lanes (two-pass,
+// fp32 statistics, biased variance), result rounded to bf16 and packed.
+__device__ __forceinline__ u32x4 ln_row16(const float (&x)[8], const float (&gam)[8],
+                                          const float (&bet)[8], float eps) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) s += x[i];
+    const float mean = row16_sum(s) * (1.0f / kC);
+    float d[8], q = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { d[i] = x[i] - mean; q += d[i] * d[i]; }
+    const float rstd = __builtin_amdgcn_rsqf(row16_sum(q) * (1.0f / kC) + eps);
+    u32x4 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        float a = d[2 * i] * rstd * gam[2 * i] + bet[2 * i];
+        float b = d[2 * i + 1] * rstd * gam[2 * i + 1] + bet[2 * i + 1];
+        o[i] = pack_bf16(a, b);
+    }
+    return o;
+}
+
+}  // namespace kfh

@@ -1,0 +1,286 @@
+// Triangle multiplication, input and output phases (C = D = 128).
+//
+// Follows the math of the reference's torch path
+// (src/kfold/model/primitives/triangle_multiplication.py:212-229 outgoing, :296-313
+// incoming):
+//     xn  = LN_in(z)
+//     ab  = (Wp_in xn) * sigmoid(Wg_in xn) * mask          a = first D channels, b = last D
+//     y   = sum_k a[i,k] b[j,k]   (outgoing)   |   sum_k a[k,i] b[k,j]   (incoming)
+//     out = (Wp_out LN_out(y)) * sigmoid(Wg_out xn)
+//
+// trimul_in_kernel   z -> channel-major planes ab[2D][Np][Np] (bf16, zero padded) + gate
+// contract_kernel    (contract.hip) per channel d:  Y_d = A_d * B_d^T
+// trimul_out_kernel  planes y[D][Np][Np] -> LN_out -> Wp_out -> * gate (+ residual) -> out
+//
+// For the incoming direction the input phase walks z down a column and stores the plane
+// transposed (plane[d][i][k] = ab[k,i,d]), so the contraction is the same NT product.
+#include "kernels.hpp"
+
+namespace kfh {
+
+constexpr int kTileP = 256;   // positions per workgroup in the input phase (64 per wavefront)
+
+template <int IO>
+__global__ __launch_bounds__(256) void trimul_in_kernel(
+    const void* __restrict__ z, const uint8_t* __restrict__ mask, const char* __restrict__ blob,
+    uint16_t* __restrict__ planes, uint16_t* __restrict__ gate, int N, int Np, int incoming,
+    float eps) {
+    // staged LayerNorm rows first, then two 16 KiB weight buffers over the same memory
+    __shared__ __attribute__((aligned(16))) char smem[kTileP * kXS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int line = blockIdx.y, t0 = blockIdx.x * kTileP;
+    const size_t plane_sz = (size_t)Np * Np;
+
+    if (line >= N) {   // padded line: zeros in every plane
+        const int t = t0 + 2 * (tid & 127);
+        if (t < Np) {
+            for (int ch = tid >> 7; ch < 2 * kC; ch += 2)
+                *reinterpret_cast<uint32_t*>(planes + ch * plane_sz + (size_t)line * Np + t) = 0u;
+        }
+        return;
+    }
+
+    // ---- phase A: load 256 rows, LayerNorm, stage as bf16 ---------------------------------
+    {
+        const float* lnp = reinterpret_cast<const float*>(blob + kTmLnOff);
+        const int r16 = tid >> 4, ch = tid & 15;
+        float gam[8], bet[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) { gam[i] = lnp[ch * 8 + i]; bet[i] = lnp[kC + ch * 8 + i]; }
+#pragma unroll 2
+        for (int it = 0; it < kTileP / 16; ++it) {
+            const int row = it * 16 + r16, t = t0 + row;
+            float x[8];
+            if (t < N) {
+                const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
+                load8<IO>(z, pos * kC + ch * 8, x);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = 0.f;
+            }
+            *reinterpret_cast<u32x4*>(smem + row * kXS + ch * 16) = ln_row16(x, gam, bet, eps);
+        }
+    }
+    __syncthreads();
+
+    // ---- phase B: fragments of this wavefront's 64 positions; lane col <-> positions 2col+pb
+    bf16x8 xf[2][kKS];
+    float mk[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int row = wave * 64 + 2 * col + pb, t = t0 + row;
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks) xf[pb][ks] = lds_frag(smem, row, ks, half);
+        mk[pb] = 0.f;
+        if (t < N) {
+            const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
+            mk[pb] = mask[pos] ? 1.f : 0.f;
+        }
+    }
+    __syncthreads();
+
+    // ---- phase C: 10 steps of two 32-column weight blocks, weights double-buffered in LDS --
+    constexpr int NSTEP = 10;
+    const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTmInOff);
+    u32x4 pre[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) pre[i] = wsrc[i * 256 + tid];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) reinterpret_cast<u32x4*>(smem)[i * 256 + tid] = pre[i];
+    __syncthreads();
+
+    const int tpos = t0 + wave * 64 + 2 * col;
+    for (int s = 0; s < NSTEP; ++s) {
+        const char* wcur = smem + (s & 1) * 16384;
+        if (s + 1 < NSTEP) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) pre[i] = wsrc[(s + 1) * 1024 + i * 256 + tid];
+        }
+        f32x16 acc[2][2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[b][pb][v] = 0.f;
+
+        if (s < 8) {
+            // a|b channels 32s..32s+31: weights as the A operand (rows = channels)
+#pragma unroll
+            for (int ks = 0; ks < kKS; ++ks) {
+                const bf16x8 w0 = *reinterpret_cast<const bf16x8*>(wcur + ks * 1024 + lane * 16);
+                const bf16x8 w1 = *reinterpret_cast<const bf16x8*>(wcur + 8192 + ks * 1024 + lane * 16);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) {
+                    acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
+                    acc[1][pb] = mfma32(w1, xf[pb][ks], acc[1][pb]);
+                }
+            }
+            if (tpos < Np) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int chn = s * 32 + acc_row(v, half);
+                    const float a0 = acc[0][0][v] * sigmoidf_fast(acc[1][0][v]) * mk[0];
+                    const float a1 = acc[0][1][v] * sigmoidf_fast(acc[1][1][v]) * mk[1];
+                    *reinterpret_cast<uint32_t*>(planes + chn * plane_sz + (size_t)line * Np + tpos) =
+                        pack_bf16(a0, a1);
+                }
+            }
+        } else {
+            // output gate channels 64gs + 2col + b: activations as the A operand (rows = positions)
+            const int gs = s - 8;
+#pragma unroll
+            for (int ks = 0; ks < kKS; ++ks) {
+                const bf16x8 w0 = *reinterpret_cast<const bf16x8*>(wcur + ks * 1024 + lane * 16);
+                const bf16x8 w1 = *reinterpret_cast<const bf16x8*>(wcur + 8192 + ks * 1024 + lane * 16);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) {
+                    acc[0][pb] = mfma32(xf[pb][ks], w0, acc[0][pb]);
+                    acc[1][pb] = mfma32(xf[pb][ks], w1, acc[1][pb]);
+                }
+            }
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int t = t0 + wave * 64 + 2 * acc_row(v, half) + pb;
+                    if (t < N) {
+                        const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
+                        *reinterpret_cast<uint32_t*>(gate + pos * kC + 64 * gs + 2 * col) =
+                            pack_bf16(sigmoidf_fast(acc[0][pb][v]), sigmoidf_fast(acc[1][pb][v]));
+                    }
+                }
+            }
+        }
+        if (s + 1 < NSTEP) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                reinterpret_cast<u32x4*>(smem + ((s + 1) & 1) * 16384)[i * 256 + tid] = pre[i];
+        }
+        __syncthreads();
+    }
+}
+
+void launch_trimul_in(const void* z, int io_dtype, const uint8_t* mask, const char* blob,
+                      uint16_t* planes, uint16_t* gate, int N, int Np, int incoming, float eps,
+                      hipStream_t stream) {
+    dim3 grid((Np + kTileP - 1) / kTileP, Np), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(trimul_in_kernel<KFH_F32>, grid, block, 0, stream, z, mask, blob, planes,
+                           gate, N, Np, incoming, eps);
+    else
+        hipLaunchKernelGGL(trimul_in_kernel<KFH_BF16>, grid, block, 0, stream, z, mask, blob, planes,
+                           gate, N, Np, incoming, eps);
+}
+
+// -----------------------------------------------------------------------------------------
+// output phase: 128 positions of one row i per workgroup, 32 per wavefront
+// -----------------------------------------------------------------------------------------
+template <int IO>
+__global__ __launch_bounds__(256) void trimul_out_kernel(
+    const uint16_t* __restrict__ planes_y, const uint16_t* __restrict__ gate,
+    const char* __restrict__ blob, const void* residual, void* out, int N, int Np, float eps) {
+    __shared__ __attribute__((aligned(16))) char yt[kC * kXS];   // [d][128 positions] bf16
+    __shared__ float lnw[2 * kC];                                // LN_out gamma, beta
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int i = blockIdx.y, j0 = blockIdx.x * 128;
+    {
+        const int r16 = tid >> 4, ch = tid & 15;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int d = it * 16 + r16;
+            const u32x4 v = *reinterpret_cast<const u32x4*>(
+                planes_y + ((size_t)d * Np + i) * Np + j0 + ch * 8);
+            *reinterpret_cast<u32x4*>(yt + d * kXS + ch * 16) = v;
+        }
+        lnw[tid] = reinterpret_cast<const float*>(blob + kTmLnOff)[2 * kC + tid];
+    }
+    __syncthreads();
+
+    // lane (col, half) owns position 32*wave + col and channels d = 64*half + 0..63 (K_HALF)
+    const int p = 32 * wave + col;
+    float y[64];
+    float s = 0.f;
+#pragma unroll
+    for (int dd = 0; dd < 64; ++dd) {
+        const uint16_t w = *reinterpret_cast<const uint16_t*>(yt + (64 * half + dd) * kXS + p * 2);
+        y[dd] = __uint_as_float((uint32_t)w << 16);
+        s += y[dd];
+    }
+    const float mean = xhalf_sum(s) * (1.0f / kC);
+    float q = 0.f;
+#pragma unroll
+    for (int dd = 0; dd < 64; ++dd) { y[dd] -= mean; q += y[dd] * y[dd]; }
+    const float rstd = __builtin_amdgcn_rsqf(xhalf_sum(q) * (1.0f / kC) + eps);
+    bf16x8 yf[kKS];
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) {
+        u32x4 w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int d0 = 64 * half + 8 * ks + 2 * e;
+            const float a = y[8 * ks + 2 * e] * rstd * lnw[d0] + lnw[kC + d0];
+            const float b = y[8 * ks + 2 * e + 1] * rstd * lnw[d0 + 1] + lnw[kC + d0 + 1];
+            w[e] = pack_bf16(a, b);
+        }
+        yf[ks] = __builtin_bit_cast(bf16x8, w);
+    }
+
+    f32x16 acc[4];
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[nb][v] = 0.f;
+    const bf16x8* wo = reinterpret_cast<const bf16x8*>(blob + kTmOutOff);
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks)
+            acc[nb] = mfma32(yf[ks], wo[(nb * kKS + ks) * 64 + lane], acc[nb]);
+
+    // block nb, lane col <-> channel 4*col + nb (ROW_INTERLEAVE4): 8 or 16 contiguous bytes per lane
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        const int j = j0 + 32 * wave + acc_row(v, half);
+        if (j < N) {
+            const size_t e0 = ((size_t)i * N + j) * kC + 4 * col;
+            const u32x2 g = *reinterpret_cast<const u32x2*>(gate + e0);
+            float o0 = acc[0][v] * bf16_lo(g[0]);
+            float o1 = acc[1][v] * bf16_hi(g[0]);
+            float o2 = acc[2][v] * bf16_lo(g[1]);
+            float o3 = acc[3][v] * bf16_hi(g[1]);
+            if constexpr (IO == KFH_BF16) {
+                if (residual) {
+                    const u32x2 r = *reinterpret_cast<const u32x2*>(
+                        static_cast<const uint16_t*>(residual) + e0);
+                    o0 += bf16_lo(r[0]); o1 += bf16_hi(r[0]); o2 += bf16_lo(r[1]); o3 += bf16_hi(r[1]);
+                }
+                u32x2 o = {pack_bf16(o0, o1), pack_bf16(o2, o3)};
+                *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
+            } else {
+                if (residual) {
+                    const f32x4 r = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
+                    o0 += r[0]; o1 += r[1]; o2 += r[2]; o3 += r[3];
+                }
+                f32x4 o = {o0, o1, o2, o3};
+                *reinterpret_cast<f32x4*>(static_cast<float*>(out) + e0) = o;
+            }
+        }
+    }
+}
+
+void launch_trimul_out(const uint16_t* planes_y, const uint16_t* gate, const char* blob,
+                       const void* residual, void* out, int io_dtype, int N, int Np, float eps,
+                       hipStream_t stream) {
+    dim3 grid((N + 127) / 128, N), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(trimul_out_kernel<KFH_F32>, grid, block, 0, stream, planes_y, gate, blob,
+                           residual, out, N, Np, eps);
+    else
+        hipLaunchKernelGGL(trimul_out_kernel<KFH_BF16>, grid, block, 0, stream, planes_y, gate, blob,
+                           residual, out, N, Np, eps);
+}
+
+}  // namespace kfh

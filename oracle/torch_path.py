@@ -1,0 +1,377 @@
+"""fp32 torch restatement of the reference's *torch* backend for the hot path.
+
+TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).
+
+Every class keeps the reference's parameter names so that a ``state_dict`` moves
+between the reference modules, these oracle modules and the product modules
+unchanged.  Each ``forward`` cites the reference lines it follows; paths are
+relative to the reference's ``src/kfold``.
+
+How each function is pinned (no reference-held vectors exist for this path, the
+reference ships no tests):
+
+* ``layer_norm``/``linear``/softmax: library routines, checked against closed
+  forms in ``tests/test_oracle_pins.py``;
+* triangle multiplication, triangle attention, pair-bias attention: checked
+  against fp64 pure-Python loop restatements of the index formulas
+  (``oracle/brute.py``) on tiny sizes, plus closed forms (zero gate weights give
+  a 0.5 gate, zero query weights give uniform attention, single valid key
+  returns that key's value) and invariants (ending == transpose of starting on
+  the transposed input, incoming == outgoing contraction on the transposed
+  input, token-permutation equivariance, crop-vs-pad invariance);
+* block wiring (residual order, in-place adds, final mask): checked by
+  recomposing the block from the individually pinned pieces.
+"""
+
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+
+# ---------------------------------------------------------------------------
+# leaf layers
+# ---------------------------------------------------------------------------
+class LayerNorm(nn.Module):
+    """model/primitives/normalization.py:22-91 — statistics in fp32, cast back."""
+
+    def __init__(self, dim: int, create_scale: bool = True, create_offset: bool = True,
+                 eps: float = 1e-5):
+        super().__init__()
+        self.normalized_shape = dim
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim)) if create_scale else None
+        self.bias = nn.Parameter(torch.zeros(dim)) if create_offset else None
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        y = F.layer_norm(x.float(), (self.normalized_shape,), self.weight, self.bias, self.eps)
+        return y.to(x.dtype)
+
+
+class Linear(nn.Module):
+    """model/primitives/linear.py:22-107 — ``y = x W^T (+ b)``, ``W`` is [out, in]."""
+
+    def __init__(self, c_in: int, c_out: int, bias: bool = True):
+        super().__init__()
+        self.weight = nn.Parameter(torch.zeros(c_out, c_in))
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(c_out))
+        else:
+            self.register_parameter("bias", None)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return F.linear(x, self.weight, self.bias)
+
+
+class LinearNoBias(Linear):
+    """model/primitives/linear.py:110-126."""
+
+    def __init__(self, c_in: int, c_out: int):
+        super().__init__(c_in, c_out, bias=False)
+
+
+class SwiGLU(nn.Module):
+    """model/primitives/activation.py:20-29 — ``silu(first half) * second half``."""
+
+    def __init__(self, c_in: int, c_out: int):
+        super().__init__()
+        self.linear = LinearNoBias(c_in, 2 * c_out)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        u, v = self.linear(x).chunk(2, dim=-1)
+        return F.silu(u) * v
+
+
+class Transition(nn.Module):
+    """model/layers/folding/transition.py:20-68."""
+
+    def __init__(self, channel: int, expansion_factor: int):
+        super().__init__()
+        self.model_dim = channel * expansion_factor
+        self.layernorm = LayerNorm(channel)
+        self.swiglu = SwiGLU(channel, self.model_dim)
+        self.linear_out = LinearNoBias(self.model_dim, channel)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.linear_out(self.swiglu(self.layernorm(x)))
+
+
+class AdaLN(nn.Module):
+    """model/primitives/normalization.py:94-125."""
+
+    def __init__(self, channel_a: int, channel_s: int):
+        super().__init__()
+        self.layernorm_a = LayerNorm(channel_a, create_scale=False, create_offset=False)
+        self.layernorm_s = LayerNorm(channel_s, create_scale=True, create_offset=False)
+        self.linear_g = Linear(channel_s, channel_a)
+        self.linear_bias = LinearNoBias(channel_s, channel_a)
+
+    def forward(self, a: torch.Tensor, s: torch.Tensor) -> torch.Tensor:
+        a = self.layernorm_a(a)
+        s = self.layernorm_s(s)
+        return torch.sigmoid(self.linear_g(s)) * a + self.linear_bias(s)
+
+
+# ---------------------------------------------------------------------------
+# triangle multiplication
+# ---------------------------------------------------------------------------
+class _TriangleMultiplication(nn.Module):
+    """model/primitives/triangle_multiplication.py:148-313 (torch branch)."""
+
+    direction = ""
+
+    def __init__(self, dim: int = 128, kernel_backend: str = "torch"):
+        super().__init__()
+        self.kernel_backend = kernel_backend
+        self.layernorm_in = LayerNorm(dim)
+        self.linear_p_in = LinearNoBias(dim, 2 * dim)
+        self.linear_g_in = LinearNoBias(dim, 2 * dim)
+        self.layernorm_out = LayerNorm(dim)
+        self.linear_p_out = LinearNoBias(dim, dim)
+        self.linear_g_out = LinearNoBias(dim, dim)
+
+    def forward(self, x: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+        # :212-229 (outgoing) / :296-313 (incoming)
+        xn = self.layernorm_in(x)
+        ab = self.linear_p_in(xn) * torch.sigmoid(self.linear_g_in(xn))
+        ab = ab * mask.unsqueeze(-1)
+        a, b = torch.chunk(ab.float(), 2, dim=-1)
+        if self.direction == "outgoing":
+            y = torch.einsum("bikd,bjkd->bijd", a, b)      # :224
+        else:
+            y = torch.einsum("bkid,bkjd->bijd", a, b)      # :308
+        return self.linear_p_out(self.layernorm_out(y)) * torch.sigmoid(self.linear_g_out(xn))
+
+
+class TriangleMultiplicationOutgoing(_TriangleMultiplication):
+    direction = "outgoing"
+
+
+class TriangleMultiplicationIncoming(_TriangleMultiplication):
+    direction = "incoming"
+
+
+# ---------------------------------------------------------------------------
+# triangle attention
+# ---------------------------------------------------------------------------
+class MultiHeadAttention(nn.Module):
+    """model/primitives/triangle_attention.py:172-335 (torch branch)."""
+
+    def __init__(self, c_q: int, c_k: int, c_v: int, c_hidden: int, no_heads: int,
+                 gating: bool = True, inf: float = 1e9):
+        super().__init__()
+        self.c_hidden = c_hidden
+        self.no_heads = no_heads
+        self.inf = inf
+        self.linear_q = LinearNoBias(c_q, c_hidden * no_heads)
+        self.linear_k = LinearNoBias(c_k, c_hidden * no_heads)
+        self.linear_v = LinearNoBias(c_v, c_hidden * no_heads)
+        self.linear_o = LinearNoBias(c_hidden * no_heads, c_q)
+        self.linear_g = LinearNoBias(c_q, c_hidden * no_heads) if gating else None
+
+    def forward(self, q_x, kv_x, tri_bias, mask):
+        h = self.no_heads
+        # :246-267 — project, split heads, move heads in front of the sequence axis
+        q = self.linear_q(q_x).unflatten(-1, (h, -1)).transpose(-2, -3)
+        k = self.linear_k(kv_x).unflatten(-1, (h, -1)).transpose(-2, -3)
+        v = self.linear_v(kv_x).unflatten(-1, (h, -1)).transpose(-2, -3)
+        q = q / math.sqrt(self.c_hidden)
+        # :328-330, :132-152 — logits = q k^T, then += mask bias, then += pair bias
+        logits = torch.matmul(q, k.transpose(-1, -2))
+        logits = logits + (-self.inf) * (~mask.bool()).to(q.dtype)
+        logits = logits + tri_bias
+        o = torch.matmul(torch.softmax(logits, dim=-1), v).transpose(-2, -3)
+        # :269-283 — gate with sigmoid(linear_g(q_x)), merge heads, project
+        if self.linear_g is not None:
+            g = torch.sigmoid(self.linear_g(q_x)).unflatten(-1, (h, -1))
+            o = o * g
+        return self.linear_o(o.flatten(-2))
+
+
+class TriangleAttention(nn.Module):
+    """model/primitives/triangle_attention.py:338-434 (torch branch).
+
+    ``row_chunk`` bounds the [rows, H, N, N] logits held at once; rows are
+    independent so the result does not depend on it.
+    """
+
+    def __init__(self, c_in: int, no_heads: int, starting: bool, inf: float = 1e9,
+                 kernel_backend: str = "torch", row_chunk: int | None = None):
+        super().__init__()
+        assert c_in % no_heads == 0
+        self.c_in = c_in
+        self.c_hidden = c_in // no_heads
+        self.no_heads = no_heads
+        self.starting = starting
+        self.inf = inf
+        self.kernel_backend = kernel_backend
+        self.row_chunk = row_chunk
+        self.layer_norm = LayerNorm(c_in)
+        self.linear = LinearNoBias(c_in, no_heads)
+        # the reference does not forward ``inf`` to the inner attention (:366-373): it keeps 1e9
+        self.mha = MultiHeadAttention(c_in, c_in, c_in, self.c_hidden, no_heads)
+
+    def forward(self, x: torch.Tensor, mask: torch.Tensor | None = None) -> torch.Tensor:
+        if mask is None:                                     # :394-398
+            mask = x.new_ones(x.shape[:-1])
+        if not self.starting:                                # :400-402
+            x = x.transpose(-2, -3)
+            mask = mask.transpose(-1, -2)
+        x = self.layer_norm(x)                               # :411
+        # :416-422 — bias [*, I, J, H] -> [*, 1, H, I, J]; here I plays "query", J "key"
+        bias = self.linear(x).movedim(-1, -3).unsqueeze(-4)
+        mask5 = mask[..., :, None, None, :]                  # :414  [*, I, 1, 1, J]
+        n_rows = x.shape[-3]
+        step = self.row_chunk or n_rows
+        outs = []
+        for r0 in range(0, n_rows, step):
+            xs = x[..., r0:r0 + step, :, :]
+            outs.append(self.mha(xs, xs, bias, mask5[..., r0:r0 + step, :, :, :]))
+        out = torch.cat(outs, dim=-3)
+        if not self.starting:                                # :431-432
+            out = out.transpose(-2, -3)
+        return out
+
+
+class TriangleAttentionStartingNode(TriangleAttention):
+    def __init__(self, c_in: int, no_heads: int, inf: float = 1e9,
+                 kernel_backend: str = "torch", row_chunk: int | None = None):
+        super().__init__(c_in, no_heads, True, inf, kernel_backend, row_chunk)
+
+
+class TriangleAttentionEndingNode(TriangleAttention):
+    def __init__(self, c_in: int, no_heads: int, inf: float = 1e9,
+                 kernel_backend: str = "torch", row_chunk: int | None = None):
+        super().__init__(c_in, no_heads, False, inf, kernel_backend, row_chunk)
+
+
+# ---------------------------------------------------------------------------
+# pair-bias attention
+# ---------------------------------------------------------------------------
+def torch_attention_pair_bias(module, x_q, x_k, pair_bias, mask):
+    """model/primitives/attention.py:75-94 + :239-271 + :122-168 (``"torch"`` kernel)."""
+    h, dh = module.num_heads, module.head_dim
+    q = module.linear_q(x_q).unflatten(-1, (h, dh)).transpose(-2, -3)
+    k = module.linear_k(x_k).unflatten(-1, (h, dh)).transpose(-2, -3)
+    v = module.linear_v(x_k).unflatten(-1, (h, dh)).transpose(-2, -3)
+    bias = pair_bias - module.inf * (~mask.bool()).float()[..., None, None, :]   # :255-257
+    scale = 1.0 / math.sqrt(dh)
+    logits = torch.einsum("...qc,...kc->...qk", q.float() * scale, k.float())    # :156
+    logits = logits + bias.float()
+    attn = torch.softmax(logits, dim=-1).to(v.dtype)
+    av = torch.einsum("...qk,...kc->...qc", attn, v)                              # :166
+    av = av.transpose(-2, -3).reshape(x_q.shape)                                  # :267
+    g = torch.sigmoid(F.linear(x_q, module.linear_g.weight, module.linear_g.bias))
+    return F.linear(g * av, module.linear_out.weight, module.linear_out.bias)    # :269-270
+
+
+class SelfAttentionPairBias(nn.Module):
+    """model/layers/folding/attention_pair_bias.py:30-158."""
+
+    def __init__(self, channel_a: int, num_heads: int, channel_s: int | None,
+                 call_site: str = "confidence", inf: float = 1e9, kernel_backend: str = "torch"):
+        super().__init__()
+        assert channel_a % num_heads == 0
+        if call_site not in {"diffusion_global", "confidence"}:
+            raise ValueError(f"Unsupported self APB call site: {call_site!r}")
+        self.channel_a = channel_a
+        self.num_heads = num_heads
+        self.head_dim = channel_a // num_heads
+        self.inf = inf
+        self.call_site = call_site
+        self.kernel_backend = kernel_backend
+        self.use_single_conditioning = channel_s is not None
+        self.linear_q = Linear(channel_a, channel_a)
+        self.linear_k = LinearNoBias(channel_a, channel_a)
+        self.linear_v = LinearNoBias(channel_a, channel_a)
+        self.linear_g = LinearNoBias(channel_a, channel_a)
+        self.linear_out = LinearNoBias(channel_a, channel_a)
+        if self.use_single_conditioning:
+            self.adaln_a = AdaLN(channel_a, channel_s)
+            self.linear_ada_out = Linear(channel_s, channel_a)
+        else:
+            self.layernorm_a = LayerNorm(channel_a)
+
+    def forward(self, a, s, pair_bias, mask):
+        if self.use_single_conditioning:
+            a = self.adaln_a(a, s)
+        else:
+            assert s is None
+            a = self.layernorm_a(a)
+        a = torch_attention_pair_bias(self, a, a, pair_bias, mask)
+        if self.use_single_conditioning:
+            a = torch.sigmoid(self.linear_ada_out(s)) * a                         # :155-157
+        return a
+
+
+# ---------------------------------------------------------------------------
+# blocks
+# ---------------------------------------------------------------------------
+class PairformerBlock(nn.Module):
+    """model/modules/apo_module.py:107-172, eval mode (dropout is the identity)."""
+
+    def __init__(self, channel_z: int = 128, num_tri_heads: int = 4,
+                 row_chunk: int | None = None):
+        super().__init__()
+        self.tri_mul_out = TriangleMultiplicationOutgoing(channel_z)
+        self.tri_mul_in = TriangleMultiplicationIncoming(channel_z)
+        self.tri_att_start = TriangleAttentionStartingNode(channel_z, num_tri_heads,
+                                                           row_chunk=row_chunk)
+        self.tri_att_end = TriangleAttentionEndingNode(channel_z, num_tri_heads,
+                                                       row_chunk=row_chunk)
+        self.transition_z = Transition(channel_z, expansion_factor=2)
+
+    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor) -> torch.Tensor:
+        # in eval mode the adds mutate the caller's tensor (primitives/utils.py:47-48)
+        z.add_(self.tri_mul_out(z, pair_mask))
+        z.add_(self.tri_mul_in(z, pair_mask))
+        z.add_(self.tri_att_start(z, pair_mask))
+        z.add_(self.tri_att_end(z, pair_mask))
+        z.add_(self.transition_z(z))
+        return z * pair_mask[..., None]
+
+
+class PairSingleBlock(nn.Module):
+    """One Pairformer block with a single track, as the benchmark configs define it.
+
+    Pair track = ``PairformerBlock`` (modules/apo_module.py:145-172); single track =
+    the part of ``ConfidencePairSingleBlock.forward`` after its pair block
+    (modules/confidence_head.py:161-175): ``bias = linear_pair_bias(LN(z))`` moved to
+    [B, H, L, L], ``s += SelfAttentionPairBias(s, None, bias, mask)``,
+    ``s += Transition_4(s)``.
+    """
+
+    def __init__(self, channel_s: int = 384, channel_z: int = 128, num_heads: int = 16,
+                 num_tri_heads: int = 4, row_chunk: int | None = None):
+        super().__init__()
+        self.pair_block = PairformerBlock(channel_z, num_tri_heads, row_chunk=row_chunk)
+        self.layernorm_z = LayerNorm(channel_z)
+        self.linear_pair_bias = LinearNoBias(channel_z, num_heads)
+        self.attention = SelfAttentionPairBias(channel_s, num_heads, None, call_site="confidence")
+        self.transition = Transition(channel_s, expansion_factor=4)
+
+    def forward(self, z, s, pair_mask, mask):
+        z = self.pair_block(z, pair_mask)
+        pair_bias = self.linear_pair_bias(self.layernorm_z(z)).movedim(-1, -3)
+        s.add_(self.attention(s, None, pair_bias, mask))
+        s.add_(self.transition(s))
+        return z, s
+
+
+class PairformerTrunk(nn.Module):
+    """A stack of ``PairSingleBlock`` (plain loop at inference, utils/checkpointing.py:85-86)."""
+
+    def __init__(self, num_blocks: int, channel_s: int = 384, channel_z: int = 128,
+                 num_heads: int = 16, num_tri_heads: int = 4, row_chunk: int | None = None):
+        super().__init__()
+        self.blocks = nn.ModuleList(
+            PairSingleBlock(channel_s, channel_z, num_heads, num_tri_heads, row_chunk)
+            for _ in range(num_blocks))
+
+    def forward(self, z, s, pair_mask, mask):
+        for blk in self.blocks:
+            z, s = blk(z, s, pair_mask, mask)
+        return z, s

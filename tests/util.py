@@ -1,0 +1,34 @@
+"""Shared helpers for the parity tests."""
+
+from __future__ import annotations
+
+import torch
+
+# north-star tolerances of the bf16 HIP path against the fp32 oracle
+MAX_ABS = 2e-2
+MEAN_ABS = 2e-3
+# this repo's own, sharper gate: relative Frobenius error of a bf16 pipeline
+REL_FRO = 2e-2
+
+
+def errors(out: torch.Tensor, ref: torch.Tensor) -> dict:
+    o = out.detach().float().cpu()
+    r = ref.detach().float().cpu()
+    d = (o - r).abs()
+    return {
+        "max_abs": d.max().item() if d.numel() else 0.0,
+        "mean_abs": d.mean().item() if d.numel() else 0.0,
+        "rel_fro": ((o - r).norm() / r.norm().clamp_min(1e-30)).item() if d.numel() else 0.0,
+        "finite": bool(torch.isfinite(o).all()),
+    }
+
+
+def assert_close(out, ref, what="", max_abs=MAX_ABS, mean_abs=MEAN_ABS, rel_fro=REL_FRO):
+    e = errors(out, ref)
+    msg = f"{what}: {e}"
+    assert e["finite"], msg
+    assert e["max_abs"] <= max_abs, msg
+    assert e["mean_abs"] <= mean_abs, msg
+    if rel_fro is not None:
+        assert e["rel_fro"] <= rel_fro, msg
+    return e
