@@ -75,6 +75,33 @@ int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, con
                        void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                        int direction, float eps, int io_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Triangle attention around the starting / ending node (Algorithms 14/15).
+ * Replaces kernels/triton/triangle_attention/ops.py:24 `precompute` and :56 `forward` as
+ * called from model/primitives/triangle_attention.py:63-129 (`triton_triangular_attn`);
+ * math of the torch path at :375-434, :246-335, :132-152.
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_triattn_packed_bytes(int C, int H);
+
+/* ln_* [C]; q_w, k_w, v_w, g_w [H*Dh, C] (mha.linear_{q,k,v,g}); bias_w [H, C] (`linear`);
+ * o_w [C, H*Dh] (mha.linear_o).  The 1/sqrt(Dh) query scale is folded in here. */
+int kfh_triattn_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* k_w,
+                     const void* v_w, const void* g_w, const void* bias_w, const void* o_w,
+                     int w_dtype, int C, int H, void* blob, void* stream);
+
+size_t kfh_triattn_workspace_bytes(int N, int C, int H);
+
+/* out = (residual or 0) + TriangleAttention{Starting,Ending}Node(x, mask).
+ * x, out, residual: [B, N, N, C]; mask: [B, N, N] bytes (mask[b,i,k] gates key k of row i;
+ * for `ending` != 0 the op runs on the (i,j)-transposed x and mask and transposes the
+ * result back, without materialising any transpose).  Masked keys get probability exactly
+ * 0; a row whose keys are all masked attends uniformly over its N keys (the reference's
+ * finite -1e9 semantics, triangle_attention.py:328).  Aliasing rules as for
+ * kfh_trimul_forward. */
+int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, const void* residual,
+                        void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
+                        int H, int ending, float eps, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -3,6 +3,7 @@
 #include "../../include/kfold_hip.h"
 
 #include <cstdarg>
+#include <cmath>
 #include <cstdio>
 
 #include "kernels.hpp"
@@ -116,6 +117,101 @@ int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, con
         launch_trimul_out(planes_y, gate, bl, rb, ob, io_dtype, N, np, eps, stream);
     }
     return check_launch("trimul_forward");
+}
+
+// ------------------------------------------------------------------------------------------
+// triangle attention
+// ------------------------------------------------------------------------------------------
+namespace {
+struct TaSizes { size_t frag, bias, codes, total; int nb; };
+TaSizes ta_sizes(int N) {
+    TaSizes s;
+    s.nb = (N + 31) / 32;
+    s.frag = align_up((size_t)N * 4 * s.nb * 2048);
+    s.bias = align_up((size_t)4 * s.nb * s.nb * 4096);
+    s.codes = align_up((size_t)N * s.nb * 32);
+    s.total = 5 * s.frag + s.bias + s.codes;
+    return s;
+}
+}  // namespace
+
+size_t kfh_triattn_packed_bytes(int C, int H) {
+    return (C == kC && H == 4) ? align_up(kTaBlobBytes) : 0;
+}
+
+int kfh_triattn_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* k_w,
+                     const void* v_w, const void* g_w, const void* bias_w, const void* o_w,
+                     int w_dtype, int C, int H, void* blob, void* stream_) {
+    if (C != kC || H != 4)
+        return fail(KFH_EUNSUPPORTED, "triattn_pack: C=%d H=%d, only C=128 H=4 is built", C, H);
+    if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "triattn_pack: bad w_dtype %d", w_dtype);
+    if (!q_w || !k_w || !v_w || !g_w || !bias_w || !o_w || !blob)
+        return fail(KFH_EINVAL, "triattn_pack: null weight or blob pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* b = static_cast<char*>(blob);
+    const float qscale = kLog2e / sqrtf((float)(C / H));
+    for (int h = 0; h < 4; ++h) {
+        launch_pack_blocks(q_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, qscale,
+                           b + kTaProjOff + (2 * h) * kBlockBytes, stream);
+        launch_pack_blocks(k_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                           b + kTaProjOff + (2 * h + 1) * kBlockBytes, stream);
+        launch_pack_blocks(g_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                           b + kTaProjOff + (8 + 2 * h) * kBlockBytes, stream);
+        launch_pack_blocks(v_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                           b + kTaProjOff + (8 + 2 * h + 1) * kBlockBytes, stream);
+    }
+    launch_pack_blocks(bias_w, w_dtype, H, C, C, 0, 1, ROW_NATURAL, K_NATURAL, kLog2e,
+                       b + kTaProjOff + 16 * kBlockBytes, stream);
+    launch_fill_zero(b + kTaProjOff + 17 * kBlockBytes, kBlockBytes, stream);
+    launch_pack_blocks(o_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE4, K_ACC, 1.f, b + kTaOutOff, stream);
+    float* ln = reinterpret_cast<float*>(b + kTaLnOff);
+    launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);
+    launch_copy_f32(ln_b, w_dtype, ln + C, C, 0.f, stream);
+    return check_launch("triattn_pack");
+}
+
+size_t kfh_triattn_workspace_bytes(int N, int C, int H) {
+    if (C != kC || H != 4 || N <= 0 || N > 8192) return 0;
+    return ta_sizes(N).total;
+}
+
+int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, const void* residual,
+                        void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
+                        int H, int ending, float eps, int io_dtype, void* stream_) {
+    if (C != kC || H != 4)
+        return fail(KFH_EUNSUPPORTED, "triattn_forward: C=%d H=%d, only C=128 H=4 is built", C, H);
+    if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "triattn_forward: bad shape B=%d N=%d", B, N);
+    if (N > 8192) return fail(KFH_EUNSUPPORTED, "triattn_forward: N=%d > 8192", N);
+    if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "triattn_forward: bad io_dtype %d", io_dtype);
+    if (!x || !mask || !blob || !out || !workspace)
+        return fail(KFH_EINVAL, "triattn_forward: null pointer argument");
+    if (out == x && residual != x)
+        return fail(KFH_EINVAL, "triattn_forward: out may alias x only when residual == x");
+    const TaSizes sz = ta_sizes(N);
+    if (workspace_bytes < sz.total)
+        return fail(KFH_EINVAL, "triattn_forward: workspace %zu < %zu bytes", workspace_bytes, sz.total);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* w = static_cast<char*>(workspace);
+    TriattnWorkspace ws;
+    ws.qf = w; ws.kf = w + sz.frag; ws.vf = w + 2 * sz.frag; ws.gf = w + 3 * sz.frag;
+    ws.of = w + 4 * sz.frag;
+    ws.biasf = reinterpret_cast<float*>(w + 5 * sz.frag);
+    ws.codes = reinterpret_cast<uint8_t*>(w + 5 * sz.frag + sz.bias);
+    const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
+    for (int b = 0; b < B; ++b) {
+        const size_t off = (size_t)b * N * N * C * esz;
+        if (N % 32) {
+            // queries beyond N in the last query block have no projected bias: keep their tiles finite
+            for (int h = 0; h < 4; ++h)
+                launch_fill_zero(ws.biasf + (((size_t)h * sz.nb + (sz.nb - 1)) * sz.nb) * 1024,
+                                 (size_t)sz.nb * 4096, stream);
+        }
+        launch_triattn(static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N,
+                       static_cast<const char*>(blob), ws,
+                       residual ? static_cast<const char*>(residual) + off : nullptr,
+                       static_cast<char*>(out) + off, N, ending, eps, stream);
+    }
+    return check_launch("triattn_forward");
 }
 
 }  // extern "C"

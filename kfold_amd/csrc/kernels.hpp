@@ -41,4 +41,26 @@ void launch_trimul_out(const uint16_t* planes_y, const uint16_t* gate, const cha
                        const void* residual, void* out, int io_dtype, int N, int Np, float eps,
                        hipStream_t stream);
 
+// ---- triangle attention (triattn.hip) ------------------------------------------------------
+// Packed weight blob of one triangle-attention module (C = 128, 4 heads x 32):
+//   [0, 144K)     9 steps x 2 blocks: {q_h,k_h} h=0..3, {g_h,v_h} h=0..3, {pair bias, zero};
+//                 q and the pair bias are pre-multiplied by log2(e) (and q by 1/sqrt(32))
+//   [144K, 176K)  o projection, 4 blocks (ROW_INTERLEAVE4, K_ACC)
+//   [176K, +1K)   fp32: LN gamma, beta
+constexpr size_t kTaProjOff = 0;
+constexpr size_t kTaOutOff = 18 * kBlockBytes;
+constexpr size_t kTaLnOff = 22 * kBlockBytes;
+constexpr size_t kTaBlobBytes = kTaLnOff + 2 * kC * sizeof(float);
+
+struct TriattnWorkspace {
+    void *qf, *kf, *vf, *gf, *of;   // fragment buffers, N * 4 * nb * 2 KiB each
+    float* biasf;                    // 4 * nb * nb tiles of 4 KiB
+    uint8_t* codes;                  // N * nb * 32 key codes
+};
+
+void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream);
+void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
+                    const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
+                    float eps, hipStream_t stream);
+
 }  // namespace kfh

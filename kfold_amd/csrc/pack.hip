@@ -74,6 +74,20 @@ __global__ void copy_f32_kernel(const void* __restrict__ src, float* __restrict_
     dst[i] = x;
 }
 
+__global__ void fill_zero_kernel(u32x4* __restrict__ dst, size_t n16) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n16) dst[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
+// zero `bytes` (a multiple of 16) at a 16-byte aligned address with a plain kernel, so that
+// callers may record the call sequence into a HIP graph
+void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream) {
+    const size_t n16 = bytes / 16;
+    if (n16 == 0) return;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, stream,
+                       static_cast<u32x4*>(dst), n16);
+}
+
 void launch_pack_blocks(const void* src, int wdtype, int src_rows, int K, int ld, int row0,
                         int nblk, int row_mode, int k_mode, float scale, void* dst,
                         hipStream_t stream) {

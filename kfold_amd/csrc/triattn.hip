@@ -1,0 +1,441 @@
+// Triangle attention (C = 128, H = 4 heads of 32), starting and ending node.
+//
+// Math of the reference's torch path (src/kfold/model/primitives/triangle_attention.py
+// :375-434 with :246-335 and :132-152), written for x' = x (starting) or x' = x^T (ending,
+// :400-402; the result is transposed back, :431-432):
+//     xn         = LN(x')
+//     beta[h,j,k] = (W_b xn[j,k])[h]
+//     q,k,v,g    = W_{q,k,v,g} xn ,  q /= sqrt(32)
+//     L[i,h,j,k] = q[i,j,h] . k[i,k,h] + beta[h,j,k] - 1e9 * (1 - mask'[i,k])
+//     o[i,j,h]   = softmax_k(L) v[i,k,h] ;  out'[i,j] = W_o (o[i,j] * sigmoid(g[i,j]))
+//
+// triattn_proj_kernel  x' rows -> LN -> q,k,v,gate in MFMA fragment order + bias tiles + key codes
+// triattn_flash_kernel per (row, head, 32 queries): online-softmax attention over all keys
+// triattn_out_kernel   gated o fragments -> W_o -> (+ residual) -> out (transposed back)
+//
+// Fragment buffers: [row a][head h][position block of 32][k-step 0..1][lane][8 bf16], the
+// accumulator-to-fragment order of common.hpp, so the three kernels exchange MFMA operands
+// with fully coalesced 16-byte accesses and no layout conversion.  The logits are kept in
+// the exp2 domain: W_q and W_b are packed pre-multiplied by log2(e).
+//
+// Masking follows the reference's finite -1e9 semantics: for a row with at least one valid
+// key a masked key gets probability exactly 0; for a row with no valid key every real key
+// gets the same logit (q.k + beta is absorbed by -1e9 in fp32), i.e. uniform attention.
+#include "kernels.hpp"
+
+namespace kfh {
+
+constexpr int kH = 4;          // heads
+constexpr int kTileA = 256;    // positions per workgroup in proj/out kernels (64 per wavefront)
+
+__device__ __forceinline__ size_t frag_index(int a, int h, int blk, int ks, int nb, int lane) {
+    return ((((size_t)a * kH + h) * nb + blk) * 2 + ks) * 64 + lane;
+}
+
+// key codes: 0 = beyond N (padding of the last block), 1 = masked, 2 = valid
+template <int IO>
+__global__ __launch_bounds__(256) void triattn_proj_kernel(
+    const void* __restrict__ x, const uint8_t* __restrict__ mask, const char* __restrict__ blob,
+    bf16x8* __restrict__ qf, bf16x8* __restrict__ kf, bf16x8* __restrict__ vf,
+    bf16x8* __restrict__ gf, float* __restrict__ biasf, uint8_t* __restrict__ codes, int N, int nb,
+    int ending, float eps) {
+    __shared__ __attribute__((aligned(16))) char smem[kTileA * kXS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int a = blockIdx.y, t0 = blockIdx.x * kTileA;
+
+    stage_ln_rows<IO, kTileA>(smem, x, reinterpret_cast<const float*>(blob + kTaLnOff), eps, tid,
+                              [&](int row) -> long long {
+                                  const int b = t0 + row;
+                                  if (b >= N) return -1;
+                                  const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
+                                  return (long long)(pos * kC);
+                              });
+    __syncthreads();
+
+    // wavefront = 64 positions = blocks blk0, blk0+1; lane col <-> position 32*pb + col
+    const int blk0 = (t0 + wave * 64) >> 5;
+    bf16x8 xf[2][kKS];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int row = wave * 64 + 32 * pb + col;
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks) xf[pb][ks] = lds_frag(smem, row, ks, half);
+        const int b = t0 + row;
+        if (half == 0 && blk0 + pb < nb) {
+            uint8_t code = 0;
+            if (b < N) {
+                const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
+                code = mask[pos] ? 2 : 1;
+            }
+            codes[(size_t)a * nb * 32 + b] = code;
+        }
+    }
+    __syncthreads();
+
+    // 9 steps of two 32-column weight blocks (16 KiB), double-buffered in LDS:
+    //   0..3  { q_h , k_h }   both with channels as accumulator rows (weights = A operand)
+    //   4..7  { g_h , v_h }   g_h like q; v_h with positions as rows (activations = A operand)
+    //   8     { pair bias, - } rows 0..3 of the block are the 4 heads
+    const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTaProjOff);
+    u32x4 pre[4];
+    auto prefetch = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pre[i] = wsrc[s * 1024 + i * 256 + tid];
+    };
+    auto commit = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            reinterpret_cast<u32x4*>(smem + (s & 1) * 16384)[i * 256 + tid] = pre[i];
+    };
+    auto wfrag = [&](int s, int blk, int ks) {
+        return *reinterpret_cast<const bf16x8*>(smem + (s & 1) * 16384 + blk * 8192 + ks * 1024 + lane * 16);
+    };
+    auto store_frags = [&](bf16x8* dst, int h, int pb, const f32x16& c) {
+        bf16x8 f0, f1;
+        acc_to_frags(c, f0, f1);
+        dst[frag_index(a, h, blk0 + pb, 0, nb, lane)] = f0;
+        dst[frag_index(a, h, blk0 + pb, 1, nb, lane)] = f1;
+    };
+    prefetch(0);
+    commit(0);
+    __syncthreads();
+
+    for (int s = 0; s < 8; ++s) {
+        prefetch(s + 1);
+        const bool gv = s >= 4;
+        const int h = s & 3;
+        f32x16 acc[2][2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b)
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[b][pb][v] = 0.f;
+        if (!gv) {
+#pragma unroll
+            for (int ks = 0; ks < kKS; ++ks) {
+                const bf16x8 w0 = wfrag(s, 0, ks), w1 = wfrag(s, 1, ks);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) {
+                    acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
+                    acc[1][pb] = mfma32(w1, xf[pb][ks], acc[1][pb]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < kKS; ++ks) {
+                const bf16x8 w0 = wfrag(s, 0, ks), w1 = wfrag(s, 1, ks);
+#pragma unroll
+                for (int pb = 0; pb < 2; ++pb) {
+                    acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
+                    acc[1][pb] = mfma32(xf[pb][ks], w1, acc[1][pb]);
+                }
+            }
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[0][pb][v] = sigmoidf_fast(acc[0][pb][v]);
+        }
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb) {
+            if (blk0 + pb < nb) {
+                store_frags(gv ? gf : qf, h, pb, acc[0][pb]);
+                store_frags(gv ? vf : kf, h, pb, acc[1][pb]);
+            }
+        }
+        commit(s + 1);
+        __syncthreads();
+    }
+
+    {
+        // pair bias: x' position (a, b) is (query a, key b).  The heads are accumulator rows
+        // 0..3, i.e. registers v = 0..3 of the lanes with half == 0.  Scatter into the tile of
+        // (a/32, b/32) in accumulator order [group of 8 keys][lane = query + 32 * key-half][key % 4].
+        f32x16 acc[2];
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[pb][v] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks) {
+            const bf16x8 w0 = wfrag(8, 0, ks);
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) acc[pb] = mfma32(w0, xf[pb][ks], acc[pb]);
+        }
+        if (half == 0) {
+#pragma unroll
+            for (int pb = 0; pb < 2; ++pb) {
+                const int kblk = blk0 + pb;
+                if (kblk < nb) {
+                    const int kk = col;   // key index inside its block
+                    const int lane_q = (a & 31) + 32 * ((kk >> 2) & 1);
+#pragma unroll
+                    for (int h = 0; h < kH; ++h) {
+                        const size_t tile = ((size_t)h * nb + (a >> 5)) * nb + kblk;
+                        biasf[((tile * 4 + (kk >> 3)) * 64 + lane_q) * 4 + (kk & 3)] = acc[pb][h];
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// flash attention: wavefront = 32 queries of R rows for one head; workgroup = 4 adjacent
+// query blocks.  S^T[key][query] = K Q^T + bias is produced by the MFMA with the bias tile as
+// its C operand, so a lane owns 16 keys of one query: the row max and row sum need one
+// cross-half exchange, and exp2(S - m) rounded to bf16 is already the B operand of
+// O^T[d][query] += V^T[d][key] P^T[key][query].
+// ------------------------------------------------------------------------------------------
+template <int R>
+__global__ __launch_bounds__(256, 2) void triattn_flash_kernel(
+    const bf16x8* __restrict__ qf, const bf16x8* __restrict__ kf, const bf16x8* __restrict__ vf,
+    const bf16x8* __restrict__ gf, const f32x4* __restrict__ biasf,
+    const uint8_t* __restrict__ codes, bf16x8* __restrict__ of, int N, int nb, int qgroups,
+    int nchunks) {
+    __shared__ uint8_t cls_s[4][R][256];      // per wavefront: class of each key block per row
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int half = lane >> 5;
+
+    // chunk = (head, row set); all query groups of a chunk run on one XCD (ids are dealt
+    // round-robin over 8 XCDs), heads are the slowest index
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int chunk = (slot / qgroups) * 8 + xcd;
+    if (chunk >= nchunks) return;
+    const int qb = (slot % qgroups) * 4 + wave;
+    const int rowsets = (N + R - 1) / R;
+    const int h = chunk / rowsets, a0 = (chunk % rowsets) * R;
+    if (qb >= nb) return;
+
+    // ---- per row: classify key blocks (0 skip, 1 mixed, 2 all valid) ------------------------
+    bool uniform_row[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int a = min(a0 + r, N - 1);
+        const uint8_t* crow = codes + (size_t)a * nb * 32;
+        bool any_valid = false;
+        for (int base = 0; base < nb; base += 64) {
+            const int blk = base + lane;
+            int nvalid = 0, nreal = 0;
+            if (blk < nb) {
+                const u32x4* p = reinterpret_cast<const u32x4*>(crow + blk * 32);
+                const u32x4 c0 = p[0], c1 = p[1];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    nvalid += __popc(c0[i] & 0x02020202u) + __popc(c1[i] & 0x02020202u);
+                    nreal += __popc(c0[i] & 0x03030303u) + __popc(c1[i] & 0x03030303u);
+                }
+            }
+            any_valid = any_valid || (__ballot(nvalid > 0) != 0ull);
+            // provisional: 2 all valid, 1 some valid, 0x80 | (real keys present) otherwise
+            if (blk < nb)
+                cls_s[wave][r][blk] = nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal > 0 ? 0x81 : 0x80));
+        }
+        uniform_row[r] = !any_valid;
+    }
+    __builtin_amdgcn_s_waitcnt(0);   // LDS writes above are read below by the same wavefront
+    __builtin_amdgcn_wave_barrier();
+
+    bf16x8 q0[R], q1[R];
+    f32x16 o[R];
+    float m[R], l[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int a = min(a0 + r, N - 1);
+        q0[r] = qf[frag_index(a, h, qb, 0, nb, lane)];
+        q1[r] = qf[frag_index(a, h, qb, 1, nb, lane)];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[r][v] = 0.f;
+        m[r] = -1e30f;
+        l[r] = 0.f;
+    }
+
+    for (int kb = 0; kb < nb; ++kb) {
+        const f32x4* bt = biasf + (((size_t)h * nb + qb) * nb + kb) * 4 * 64 + lane;
+        f32x16 bias;
+        {
+            const f32x4 b0 = bt[0], b1 = bt[64], b2 = bt[128], b3 = bt[192];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { bias[e] = b0[e]; bias[4 + e] = b1[e]; bias[8 + e] = b2[e]; bias[12 + e] = b3[e]; }
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const int a = min(a0 + r, N - 1);
+            int cls = __builtin_amdgcn_readfirstlane((int)cls_s[wave][r][kb]);
+            const bool uni = uniform_row[r];
+            if (cls & 0x80) {                    // no valid key in this block
+                if (!(uni && (cls & 1))) continue;
+                cls = 1;                         // uniform row: masked real keys take part
+            }
+            const bf16x8 k0 = kf[frag_index(a, h, kb, 0, nb, lane)];
+            const bf16x8 k1 = kf[frag_index(a, h, kb, 1, nb, lane)];
+            const bf16x8 v0 = vf[frag_index(a, h, kb, 0, nb, lane)];
+            const bf16x8 v1 = vf[frag_index(a, h, kb, 1, nb, lane)];
+            f32x16 s = mfma32(k0, q0[r], bias);
+            s = mfma32(k1, q1[r], s);
+            if (cls != 2) {
+                // this lane's keys: 8*(v/4) + 4*half + (v%4) -> one dword of codes per group of 4
+                const uint32_t* cw = reinterpret_cast<const uint32_t*>(
+                    codes + (size_t)a * nb * 32 + kb * 32 + 4 * half);
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const uint32_t w = cw[2 * g];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t code = (w >> (8 * e)) & 0xffu;
+                        const int v = 4 * g + e;
+                        if (uni) s[v] = code == 1 ? 0.f : -INFINITY;
+                        else if (code != 2) s[v] = -INFINITY;
+                    }
+                }
+            }
+            float mx = s[0];
+#pragma unroll
+            for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+            mx = xhalf_max(mx);
+            const float m_new = fmaxf(m[r], mx);
+            const float alpha = fast_exp2(m[r] - m_new);
+            m[r] = m_new;
+            float ls = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) { s[v] = fast_exp2(s[v] - m_new); ls += s[v]; }
+            l[r] = l[r] * alpha + ls;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[r][v] *= alpha;
+            bf16x8 p0, p1;
+            acc_to_frags(s, p0, p1);
+            o[r] = mfma32(v0, p0, o[r]);
+            o[r] = mfma32(v1, p1, o[r]);
+        }
+    }
+
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (a0 + r < N) {
+            const int a = a0 + r;
+            const float inv = fast_rcp(xhalf_sum(l[r]));
+            const u32x4 g0 = __builtin_bit_cast(u32x4, gf[frag_index(a, h, qb, 0, nb, lane)]);
+            const u32x4 g1 = __builtin_bit_cast(u32x4, gf[frag_index(a, h, qb, 1, nb, lane)]);
+            f32x16 og;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                og[2 * e] = o[r][2 * e] * inv * bf16_lo(g0[e]);
+                og[2 * e + 1] = o[r][2 * e + 1] * inv * bf16_hi(g0[e]);
+                og[8 + 2 * e] = o[r][8 + 2 * e] * inv * bf16_lo(g1[e]);
+                og[8 + 2 * e + 1] = o[r][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
+            }
+            bf16x8 f0, f1;
+            acc_to_frags(og, f0, f1);
+            of[frag_index(a, h, qb, 0, nb, lane)] = f0;
+            of[frag_index(a, h, qb, 1, nb, lane)] = f1;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// output projection: out'[a][b] = W_o (gated o), 64 positions per wavefront
+// ------------------------------------------------------------------------------------------
+template <int IO>
+__global__ __launch_bounds__(256) void triattn_out_kernel(
+    const bf16x8* __restrict__ of, const char* __restrict__ blob, const void* residual, void* out,
+    int N, int nb, int ending) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int a = blockIdx.y, t0 = blockIdx.x * kTileA;
+    const int blk0 = (t0 + wave * 64) >> 5;
+    if (blk0 >= nb) return;
+    const bool two = blk0 + 1 < nb;
+
+    bf16x8 xf[2][kKS];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int blk = (pb == 0 || two) ? blk0 + pb : blk0;
+#pragma unroll
+        for (int h = 0; h < kH; ++h) {
+            xf[pb][2 * h] = of[frag_index(a, h, blk, 0, nb, lane)];
+            xf[pb][2 * h + 1] = of[frag_index(a, h, blk, 1, nb, lane)];
+        }
+    }
+    f32x16 acc[2][4];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+        for (int n = 0; n < 4; ++n)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[pb][n][v] = 0.f;
+    const bf16x8* wo = reinterpret_cast<const bf16x8*>(blob + kTaOutOff);
+#pragma unroll
+    for (int n = 0; n < 4; ++n)
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks) {
+            const bf16x8 w = wo[(n * kKS + ks) * 64 + lane];
+            acc[0][n] = mfma32(xf[0][ks], w, acc[0][n]);
+            acc[1][n] = mfma32(xf[1][ks], w, acc[1][n]);
+        }
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        if (pb == 1 && !two) break;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int b = (blk0 + pb) * 32 + acc_row(v, half);
+            if (b < N) {
+                const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
+                const size_t e0 = pos * kC + 4 * col;
+                float o0 = acc[pb][0][v], o1 = acc[pb][1][v], o2 = acc[pb][2][v], o3 = acc[pb][3][v];
+                if constexpr (IO == KFH_BF16) {
+                    if (residual) {
+                        const u32x2 r = *reinterpret_cast<const u32x2*>(
+                            static_cast<const uint16_t*>(residual) + e0);
+                        o0 += bf16_lo(r[0]); o1 += bf16_hi(r[0]); o2 += bf16_lo(r[1]); o3 += bf16_hi(r[1]);
+                    }
+                    u32x2 o = {pack_bf16(o0, o1), pack_bf16(o2, o3)};
+                    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
+                } else {
+                    if (residual) {
+                        const f32x4 r = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
+                        o0 += r[0]; o1 += r[1]; o2 += r[2]; o3 += r[3];
+                    }
+                    f32x4 o = {o0, o1, o2, o3};
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + e0) = o;
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
+                    const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
+                    float eps, hipStream_t stream) {
+    const int nb = (N + 31) / 32;
+    bf16x8* qf = static_cast<bf16x8*>(ws.qf);
+    bf16x8* kf = static_cast<bf16x8*>(ws.kf);
+    bf16x8* vf = static_cast<bf16x8*>(ws.vf);
+    bf16x8* gf = static_cast<bf16x8*>(ws.gf);
+    bf16x8* of = static_cast<bf16x8*>(ws.of);
+    dim3 grid_rows((N + kTileA - 1) / kTileA, N), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(triattn_proj_kernel<KFH_F32>, grid_rows, block, 0, stream, x, mask, blob, qf,
+                           kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+    else
+        hipLaunchKernelGGL(triattn_proj_kernel<KFH_BF16>, grid_rows, block, 0, stream, x, mask, blob,
+                           qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+
+    constexpr int R = 4;
+    const int qgroups = (nb + 3) / 4;
+    const int nchunks = kH * ((N + R - 1) / R);
+    const int nslots = ((nchunks + 7) / 8) * qgroups;
+    hipLaunchKernelGGL(triattn_flash_kernel<R>, dim3(nslots * 8), block, 0, stream, qf, kf, vf, gf,
+                       reinterpret_cast<const f32x4*>(ws.biasf), ws.codes, of, N, nb, qgroups,
+                       nchunks);
+
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, block, 0, stream, of, blob,
+                           residual, out, N, nb, ending);
+    else
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, block, 0, stream, of, blob,
+                           residual, out, N, nb, ending);
+}
+
+}  // namespace kfh

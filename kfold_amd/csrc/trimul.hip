@@ -42,26 +42,13 @@ __global__ __launch_bounds__(256) void trimul_in_kernel(
     }
 
     // ---- phase A: load 256 rows, LayerNorm, stage as bf16 ---------------------------------
-    {
-        const float* lnp = reinterpret_cast<const float*>(blob + kTmLnOff);
-        const int r16 = tid >> 4, ch = tid & 15;
-        float gam[8], bet[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) { gam[i] = lnp[ch * 8 + i]; bet[i] = lnp[kC + ch * 8 + i]; }
-#pragma unroll 2
-        for (int it = 0; it < kTileP / 16; ++it) {
-            const int row = it * 16 + r16, t = t0 + row;
-            float x[8];
-            if (t < N) {
-                const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
-                load8<IO>(z, pos * kC + ch * 8, x);
-            } else {
-#pragma unroll
-                for (int i = 0; i < 8; ++i) x[i] = 0.f;
-            }
-            *reinterpret_cast<u32x4*>(smem + row * kXS + ch * 16) = ln_row16(x, gam, bet, eps);
-        }
-    }
+    stage_ln_rows<IO, kTileP>(smem, z, reinterpret_cast<const float*>(blob + kTmLnOff), eps, tid,
+                              [&](int row) -> long long {
+                                  const int t = t0 + row;
+                                  if (t >= N) return -1;
+                                  const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
+                                  return (long long)(pos * kC);
+                              });
     __syncthreads();
 
     // ---- phase B: fragments of this wavefront's 64 positions; lane col <-> positions 2col+pb

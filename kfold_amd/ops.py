@@ -109,3 +109,56 @@ def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, dire
                                    KFH_INCOMING if direction == "incoming" else KFH_OUTGOING,
                                    float(eps), _io_dtype(zc), _stream(dev)))
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# triangle attention
+# ---------------------------------------------------------------------------------------
+def triattn_pack(ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w, device: torch.device) -> torch.Tensor:
+    L = _lib.lib()
+    C, H = q_w.shape[1], bias_w.shape[0]
+    nbytes = L.kfh_triattn_packed_bytes(C, H)
+    if nbytes == 0:
+        raise NotImplementedError(f"hip triangle attention is built for C=128, H=4; got C={C}, H={H}")
+    ws = _weights_f32(device, ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w)
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        check(L.kfh_triattn_pack(*[_ptr(w) for w in ws], KFH_F32, C, H, blob.data_ptr(),
+                                 _stream(device)))
+    return blob
+
+
+def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tensor, heads: int,
+                    starting: bool, eps: float = 1e-5, residual: torch.Tensor | None = None,
+                    out: torch.Tensor | None = None) -> torch.Tensor:
+    """``out = (residual or 0) + TriangleAttention(x, mask)`` for x [*, N, N, C]."""
+    dev = _require_cuda(x, mask, blob, residual, out)
+    N, C = x.shape[-2], x.shape[-1]
+    if x.dim() < 3 or x.shape[-3] != N:
+        raise ValueError(f"expected x of shape [*, N, N, C], got {tuple(x.shape)}")
+    B = x.numel() // (N * N * C) if x.numel() else 0
+    xc = x.contiguous()
+    if mask is None:
+        m8 = torch.ones(x.shape[:-1], dtype=torch.uint8, device=dev)
+    else:
+        m8 = _mask_bytes(mask, x.shape[:-1])
+    if out is None:
+        out = torch.empty_like(xc)
+    elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("out must be contiguous with the shape and dtype of x")
+    if residual is not None and (residual.shape != x.shape or residual.dtype != x.dtype
+                                 or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous with the shape and dtype of x")
+    if B == 0:
+        return out
+    L = _lib.lib()
+    ws_bytes = L.kfh_triattn_workspace_bytes(N, C, heads)
+    if ws_bytes == 0:
+        raise NotImplementedError(
+            f"hip triangle attention is built for C=128, H=4, N<=8192; got C={C}, H={heads}, N={N}")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(L.kfh_triattn_forward(xc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
+                                    out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C, heads,
+                                    0 if starting else 1, float(eps), _io_dtype(xc), _stream(dev)))
+    return out

@@ -6,3 +6,9 @@ from .triangle_multiplication import (  # noqa: F401
     TriangleMultiplicationOutgoing,
     hip_triangular_mult,
 )
+from .triangle_attention import (  # noqa: F401
+    TriangleAttention,
+    TriangleAttentionEndingNode,
+    TriangleAttentionStartingNode,
+    hip_triangular_attn,
+)

@@ -32,6 +32,12 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 
+def _up(x: torch.Tensor) -> torch.Tensor:
+    """The reference's ``.float()`` upcasts; fp64 (only used by this oracle's fp64 pin tests)
+    is left alone instead of being rounded down to fp32."""
+    return x.to(torch.promote_types(x.dtype, torch.float32))
+
+
 # ---------------------------------------------------------------------------
 # leaf layers
 # ---------------------------------------------------------------------------
@@ -47,7 +53,12 @@ class LayerNorm(nn.Module):
         self.bias = nn.Parameter(torch.zeros(dim)) if create_offset else None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        y = F.layer_norm(x.float(), (self.normalized_shape,), self.weight, self.bias, self.eps)
+        # the reference upcasts with ``x.float()``; fp64 inputs (used only by the fp64 pin
+        # tests of this oracle) are kept in fp64 instead of being rounded down to fp32
+        ct = torch.promote_types(x.dtype, torch.float32)
+        w = None if self.weight is None else self.weight.to(ct)
+        b = None if self.bias is None else self.bias.to(ct)
+        y = F.layer_norm(x.to(ct), (self.normalized_shape,), w, b, self.eps)
         return y.to(x.dtype)
 
 
@@ -138,7 +149,7 @@ class _TriangleMultiplication(nn.Module):
         xn = self.layernorm_in(x)
         ab = self.linear_p_in(xn) * torch.sigmoid(self.linear_g_in(xn))
         ab = ab * mask.unsqueeze(-1)
-        a, b = torch.chunk(ab.float(), 2, dim=-1)
+        a, b = torch.chunk(_up(ab), 2, dim=-1)
         if self.direction == "outgoing":
             y = torch.einsum("bikd,bjkd->bijd", a, b)      # :224
         else:
@@ -257,10 +268,10 @@ def torch_attention_pair_bias(module, x_q, x_k, pair_bias, mask):
     q = module.linear_q(x_q).unflatten(-1, (h, dh)).transpose(-2, -3)
     k = module.linear_k(x_k).unflatten(-1, (h, dh)).transpose(-2, -3)
     v = module.linear_v(x_k).unflatten(-1, (h, dh)).transpose(-2, -3)
-    bias = pair_bias - module.inf * (~mask.bool()).float()[..., None, None, :]   # :255-257
+    bias = pair_bias - module.inf * _up((~mask.bool()).to(pair_bias.dtype))[..., None, None, :]   # :255-257
     scale = 1.0 / math.sqrt(dh)
-    logits = torch.einsum("...qc,...kc->...qk", q.float() * scale, k.float())    # :156
-    logits = logits + bias.float()
+    logits = torch.einsum("...qc,...kc->...qk", _up(q) * scale, _up(k))          # :156
+    logits = logits + _up(bias)
     attn = torch.softmax(logits, dim=-1).to(v.dtype)
     av = torch.einsum("...qk,...kc->...qc", attn, v)                              # :166
     av = av.transpose(-2, -3).reshape(x_q.shape)                                  # :267

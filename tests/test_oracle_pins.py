@@ -1,0 +1,237 @@
+"""Pins for the oracle (``oracle/torch_path.py``).
+
+The reference ships no tests, golden vectors or fixtures for this path, so the oracle is
+pinned by (a) fp64 scalar-loop restatements of the index formulas on tiny sizes
+(``oracle/brute.py``), (b) closed forms and special cases, (c) invariants of the math.  Each
+check is chosen so that a plausible slip (swapped operand or index, wrong chunk half, dropped
+bias or mask term, gate taken from the wrong tensor) breaks it.
+"""
+
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import brute
+from oracle import torch_path as O
+
+
+def _rand_init(module, seed, std=0.4):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for name, p in module.named_parameters():
+            if p.dim() >= 2:
+                p.copy_(std * torch.randn(p.shape, generator=g))
+            elif name.endswith("bias"):
+                p.copy_(0.3 * torch.randn(p.shape, generator=g))
+            else:
+                p.copy_(1 + 0.3 * torch.randn(p.shape, generator=g))
+    return module.double().eval()
+
+
+def _np_params(module):
+    return {k: v.detach().double().numpy() for k, v in module.state_dict().items()}
+
+
+def _rand(shape, seed):
+    return torch.randn(*shape, generator=torch.Generator().manual_seed(seed), dtype=torch.float64)
+
+
+# ----------------------------------------------------------------------------- leaf layers
+def test_layernorm_closed_forms():
+    ln = O.LayerNorm(4)
+    with torch.no_grad():
+        ln.weight.copy_(torch.tensor([1.0, 2.0, 3.0, 4.0]))
+        ln.bias.copy_(torch.tensor([0.5, -0.5, 0.25, 0.0]))
+    # constant row -> (x - mu) = 0 -> beta
+    assert torch.allclose(ln(torch.full((2, 4), 7.0)), ln.bias.expand(2, 4), atol=1e-6)
+    # [-1, 1, -1, 1]: mu 0, biased var 1 -> x / sqrt(1 + eps)
+    x = torch.tensor([[-1.0, 1.0, -1.0, 1.0]])
+    want = x / math.sqrt(1 + 1e-5) * ln.weight + ln.bias
+    assert torch.allclose(ln(x), want, atol=1e-6)
+    # biased (1/n) variance, not 1/(n-1): [0, 0, 0, 2] has mu .5, var .75
+    x = torch.tensor([[0.0, 0.0, 0.0, 2.0]])
+    want = (x - 0.5) / math.sqrt(0.75 + 1e-5) * ln.weight + ln.bias
+    assert torch.allclose(ln(x), want, atol=1e-6)
+    # statistics are taken in fp32 even for a bf16 input, result cast back
+    xb = torch.randn(3, 4).bfloat16()
+    assert ln(xb).dtype == torch.bfloat16
+
+
+def test_transition_and_adaln_vs_brute():
+    t = _rand_init(O.Transition(6, 2), 1)
+    x = _rand((5, 6), 2)
+    assert np.allclose(t(x).detach().numpy(), brute.transition(x.numpy(), _np_params(t)), atol=1e-10)
+    a = _rand_init(O.AdaLN(6, 4), 3)
+    av, sv = _rand((5, 6), 4), _rand((5, 4), 5)
+    assert np.allclose(a(av, sv).detach().numpy(), brute.adaln(av.numpy(), sv.numpy(), _np_params(a)),
+                       atol=1e-10)
+
+
+# ----------------------------------------------------------------- triangle multiplication
+@pytest.mark.parametrize("cls,direction", [(O.TriangleMultiplicationOutgoing, "outgoing"),
+                                            (O.TriangleMultiplicationIncoming, "incoming")])
+def test_trimul_vs_brute(cls, direction):
+    m = _rand_init(cls(4), 10)
+    n = 5
+    z = _rand((1, n, n, 4), 11)
+    mask = (torch.rand(1, n, n, generator=torch.Generator().manual_seed(12)) > 0.3)
+    got = m(z, mask.double())[0].detach().numpy()
+    want = brute.tri_mul(z[0].numpy(), mask[0].numpy(), _np_params(m), direction)
+    assert np.allclose(got, want, atol=1e-9), np.abs(got - want).max()
+
+
+def test_trimul_zero_gate_weights_give_half_gates():
+    m = _rand_init(O.TriangleMultiplicationOutgoing(4), 13)
+    with torch.no_grad():
+        m.linear_g_in.weight.zero_()
+        m.linear_g_out.weight.zero_()
+    z = _rand((1, 3, 3, 4), 14)
+    ones = torch.ones(1, 3, 3, dtype=torch.float64)
+    xn = m.layernorm_in(z)
+    p = 0.5 * m.linear_p_in(xn)                      # sigmoid(0) = 1/2
+    a, b = p[..., :4], p[..., 4:]
+    y = torch.stack([torch.stack([(a[0, i] * b[0, j]).sum(0) for j in range(3)]) for i in range(3)])
+    want = 0.5 * m.linear_p_out(m.layernorm_out(y))
+    assert torch.allclose(m(z, ones)[0], want, atol=1e-10)
+
+
+def test_trimul_incoming_is_outgoing_on_transpose_when_output_gate_is_flat():
+    mo = _rand_init(O.TriangleMultiplicationOutgoing(4), 15)
+    mi = O.TriangleMultiplicationIncoming(4).double().eval()
+    with torch.no_grad():
+        mo.linear_g_out.weight.zero_()
+    mi.load_state_dict(mo.state_dict())
+    z = _rand((1, 4, 4, 4), 16)
+    mask = (torch.rand(1, 4, 4, generator=torch.Generator().manual_seed(17)) > 0.3).double()
+    assert torch.allclose(mi(z, mask), mo(z.transpose(1, 2), mask.transpose(1, 2)), atol=1e-10)
+
+
+# ---------------------------------------------------------------------- triangle attention
+@pytest.mark.parametrize("starting", [True, False])
+def test_triattn_vs_brute(starting):
+    cls = O.TriangleAttentionStartingNode if starting else O.TriangleAttentionEndingNode
+    m = _rand_init(cls(4, 2), 20)
+    n = 4
+    x = _rand((1, n, n, 4), 21)
+    mask = (torch.rand(1, n, n, generator=torch.Generator().manual_seed(22)) > 0.3)
+    mask[0, 2, :] = False                             # one fully masked row: stays finite
+    got = m(x, mask.double())[0].detach().numpy()
+    want = brute.tri_attn(x[0].numpy(), mask[0].numpy(), _np_params(m), heads=2, starting=starting)
+    assert np.isfinite(got).all()
+    assert np.allclose(got, want, atol=1e-8), np.abs(got - want).max()
+
+
+def test_triattn_ending_equals_transposed_starting_and_row_chunking():
+    ms = _rand_init(O.TriangleAttentionStartingNode(4, 2), 23)
+    me = O.TriangleAttentionEndingNode(4, 2, row_chunk=2).double().eval()
+    me.load_state_dict(ms.state_dict())
+    x = _rand((1, 5, 5, 4), 24)
+    mask = (torch.rand(1, 5, 5, generator=torch.Generator().manual_seed(25)) > 0.3).double()
+    want = ms(x.transpose(1, 2), mask.transpose(1, 2)).transpose(1, 2)
+    assert torch.allclose(me(x, mask), want, atol=1e-10)
+    assert torch.allclose(me(x, None), ms(x.transpose(1, 2), None).transpose(1, 2), atol=1e-10)
+
+
+def test_triattn_uniform_attention_and_single_key():
+    m = _rand_init(O.TriangleAttentionStartingNode(4, 2), 26)
+    with torch.no_grad():
+        m.mha.linear_q.weight.zero_()                 # no q.k term
+        m.linear.weight.zero_()                       # no pair bias
+    x = _rand((1, 3, 3, 4), 27)
+    xn = m.layer_norm(x)
+    v = m.mha.linear_v(xn)                            # [1, I, K, C]
+    g = torch.sigmoid(m.mha.linear_g(xn))
+    # all keys valid: every query of row i gets mean_k v[i, k]
+    want = m.mha.linear_o(g * v.mean(dim=2, keepdim=True))
+    assert torch.allclose(m(x, torch.ones(1, 3, 3, dtype=torch.float64)), want, atol=1e-10)
+    # only key 1 valid: every query of row i gets v[i, 1]
+    mask = torch.zeros(1, 3, 3, dtype=torch.float64)
+    mask[:, :, 1] = 1
+    want = m.mha.linear_o(g * v[:, :, 1:2])
+    assert torch.allclose(m(x, mask), want, atol=1e-10)
+
+
+# --------------------------------------------------------------------- pair-bias attention
+def test_apb_vs_brute_and_sample_sharing():
+    m = _rand_init(O.SelfAttentionPairBias(6, 2, None), 30)
+    L = 5
+    a = _rand((1, L, 6), 31)
+    bias = _rand((1, 2, L, L), 32)
+    mask = torch.tensor([[1, 1, 0, 1, 1]], dtype=torch.float64)
+    got = m(a, None, bias, mask)[0].detach().numpy()
+    an = m.layernorm_a(a)[0].detach().numpy()
+    want = brute.attention_pair_bias(an, an, bias[0].numpy(), mask[0].numpy(), _np_params(m), heads=2)
+    assert np.allclose(got, want, atol=1e-9), np.abs(got - want).max()
+    # a bias with a broadcast sample axis equals one call per sample
+    a2 = _rand((1, 3, L, 6), 33)
+    out = m(a2, None, bias[:, None], mask[:, None])
+    for s in range(3):
+        assert torch.allclose(out[:, s], m(a2[:, s], None, bias, mask), atol=1e-10)
+
+
+def test_apb_conditioned_wiring():
+    m = _rand_init(O.SelfAttentionPairBias(6, 2, 4, call_site="diffusion_global"), 34)
+    L = 4
+    a, s = _rand((1, L, 6), 35), _rand((1, L, 4), 36)
+    bias = _rand((1, 2, L, L), 37)
+    mask = torch.ones(1, L, dtype=torch.float64)
+    an = torch.from_numpy(brute.adaln(a[0].numpy(), s[0].numpy(),
+                                      {k[len("adaln_a."):]: v for k, v in _np_params(m).items()
+                                       if k.startswith("adaln_a.")}))
+    core = brute.attention_pair_bias(an.numpy(), an.numpy(), bias[0].numpy(), mask[0].numpy(),
+                                     _np_params(m), heads=2)
+    gate = torch.sigmoid(m.linear_ada_out(s))[0].detach().numpy()
+    assert np.allclose(m(a, s, bias, mask)[0].detach().numpy(), gate * core, atol=1e-9)
+
+
+# ------------------------------------------------------------------------------ invariants
+def test_token_permutation_equivariance_and_crop_invariance():
+    blk = _rand_init(O.PairformerBlock(4, 2), 40, std=0.3)
+    n, nv = 6, 4
+    z = _rand((1, n, n, 4), 41)
+    tok = torch.zeros(1, n, dtype=torch.bool)
+    tok[:, :nv] = True
+    pm = (tok[:, :, None] & tok[:, None, :]).double()
+    out = blk(z.clone(), pm)
+    # masked positions are exactly zero at block level
+    assert (out[0][~pm[0].bool()] == 0).all()
+    # cropping to the valid tokens gives the same values there
+    crop = blk(z[:, :nv, :nv].clone(), pm[:, :nv, :nv])
+    assert torch.allclose(out[:, :nv, :nv], crop, atol=1e-9)
+    # garbage in padded tokens does not leak into valid positions
+    z2 = z.clone()
+    z2[:, nv:] = 100 * _rand((1, n - nv, n, 4), 42)
+    z2[:, :, nv:] = 100 * _rand((1, n, n - nv, 4), 43)
+    assert torch.allclose(blk(z2, pm)[:, :nv, :nv], crop, atol=1e-9)
+    # permuting tokens permutes the output
+    perm = torch.tensor([2, 0, 3, 1, 5, 4])
+    zp = z[:, perm][:, :, perm]
+    pmp = pm[:, perm][:, :, perm]
+    assert torch.allclose(blk(zp.clone(), pmp), out[:, perm][:, :, perm], atol=1e-9)
+
+
+def test_block_wiring_and_in_place_residuals():
+    blk = _rand_init(O.PairSingleBlock(8, 4, 2, 2), 50, std=0.3)
+    n = 4
+    z, s = _rand((1, n, n, 4), 51), _rand((1, n, 8), 52)
+    tok = torch.tensor([[True, True, True, False]])
+    pm = (tok[:, :, None] & tok[:, None, :]).double()
+    # recompose from the individually pinned pieces
+    pb = blk.pair_block
+    zz = z.clone()
+    zz = zz + pb.tri_mul_out(zz, pm)
+    zz = zz + pb.tri_mul_in(zz, pm)
+    zz = zz + pb.tri_att_start(zz, pm)
+    zz = zz + pb.tri_att_end(zz, pm)
+    zz = zz + pb.transition_z(zz)
+    zz = zz * pm[..., None]
+    bias = blk.linear_pair_bias(blk.layernorm_z(zz)).permute(0, 3, 1, 2)
+    ss = s + blk.attention(s, None, bias, tok.double())
+    ss = ss + blk.transition(ss)
+    z_in, s_in = z.clone(), s.clone()
+    z_out, s_out = blk(z_in, s_in, pm, tok.double())
+    assert torch.allclose(z_out, zz, atol=1e-10) and torch.allclose(s_out, ss, atol=1e-10)
+    # eval-mode adds mutate the caller's tensors (the final mask multiply does not)
+    assert not torch.equal(z_in, z) and torch.equal(s_in, s_out)

@@ -1,0 +1,100 @@
+"""HIP triangle attention vs the fp32 oracle (through the C ABI, on the GPU)."""
+
+import pytest
+import torch
+
+from kfold_amd import synthetic
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _modules(starting, seed=0, ln_affine=False, std=0.02):
+    from kfold_amd import primitives as P
+    from oracle import torch_path as O
+
+    cls = "TriangleAttentionStartingNode" if starting else "TriangleAttentionEndingNode"
+    ref = getattr(O, cls)(128, 4, row_chunk=64).eval()
+    synthetic.init_weights_(ref, seed, std=std)
+    if ln_affine:
+        g = torch.Generator().manual_seed(seed + 100)
+        with torch.no_grad():
+            ref.layer_norm.weight.copy_(1 + 0.2 * torch.randn(128, generator=g))
+            ref.layer_norm.bias.copy_(0.1 * torch.randn(128, generator=g))
+    hip = getattr(P, cls)(128, 4).eval()
+    hip.load_state_dict(ref.state_dict())
+    return ref, hip.to(DEV)
+
+
+def _run(ref, hip, x, mask, dtype):
+    with torch.no_grad():
+        want = ref(x.to(dtype).float(), None if mask is None else mask.float())
+        got = hip(x.to(dtype).to(DEV), None if mask is None else mask.to(DEV))
+    assert got.dtype == dtype and got.shape == x.shape
+    return got, want
+
+
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("n,n_pad", [(64, 0), (37, 5), (130, 17), (1, 0), (256, 30)])
+def test_triattn_parity_bf16(starting, n, n_pad):
+    print(f"case triattn starting={starting} n={n} pad={n_pad}", flush=True)
+    # larger weights at n=37 make the softmax far from uniform and the bias matter
+    ref, hip = _modules(starting, ln_affine=(n == 37), std=0.1 if n == 37 else 0.02)
+    x, _, pm = synthetic.pair_inputs(n, 128, n_pad, seed=n)
+    got, want = _run(ref, hip, x, pm, torch.bfloat16)
+    # rows whose keys are all masked (padded tokens) follow the same uniform-attention rule
+    assert_close(got, want, f"triattn starting={starting} n={n}",
+                 rel_fro=4e-2 if n == 37 else 2e-2)
+
+
+@pytest.mark.parametrize("starting", [True, False])
+def test_triattn_general_mask_none_mask_f32_io(starting):
+    print(f"case triattn general mask starting={starting}", flush=True)
+    ref, hip = _modules(starting, seed=3, std=0.05)
+    n = 96
+    x, _, _ = synthetic.pair_inputs(n, 128, 0, seed=11)
+    mask = torch.rand(1, n, n, generator=torch.Generator().manual_seed(5)) > 0.3
+    mask[0, 7, :] = False     # fully masked row (starting) ...
+    mask[0, :, 9] = False     # ... and column (a fully masked "row" of the ending node)
+    got, want = _run(ref, hip, x, mask, torch.float32)
+    assert_close(got, want, f"triattn starting={starting} f32 io, general mask")
+    got, want = _run(ref, hip, x, None, torch.float32)
+    assert_close(got, want, f"triattn starting={starting} mask=None")
+
+
+@pytest.mark.parametrize("starting", [True, False])
+def test_triattn_config3_n512(starting):
+    """BASELINE config 3: N=512, key mask zeroing the last 64 tokens, bf16."""
+    print(f"case triattn config3 starting={starting}", flush=True)
+    ref, hip = _modules(starting)
+    x, _, pm = synthetic.pair_inputs(512, 128, 64, seed=0)
+    got, want = _run(ref, hip, x, pm, torch.bfloat16)
+    assert_close(got, want, f"triattn config3 starting={starting}")
+
+
+def test_triattn_ending_is_transposed_starting_batch_residual_determinism():
+    from kfold_amd import ops
+
+    print("case triattn invariants", flush=True)
+    ref, hs = _modules(True, seed=7, std=0.05)
+    _, he = _modules(False, seed=7, std=0.05)
+    n = 80
+    gen = torch.Generator().manual_seed(2)
+    x = torch.randn(2, n, n, 128, generator=gen).to(torch.bfloat16)
+    mask = torch.rand(2, n, n, generator=gen) > 0.2
+    xd, md = x.to(DEV), mask.to(DEV)
+    with torch.no_grad():
+        want = torch.stack([ref(x[b:b + 1].float(), mask[b:b + 1].float())[0] for b in range(2)])
+        got = hs(xd, md)
+        assert_close(got, want, "triattn batch")
+        assert torch.equal(got, hs(xd, md)), "run-to-run results differ"
+        # ending(x, m) == starting(x^T, m^T)^T, bit for bit: same arithmetic, different strides
+        e = he(xd, md)
+        s_t = hs(xd.transpose(1, 2).contiguous(), md.transpose(1, 2).contiguous()).transpose(1, 2)
+        assert torch.equal(e, s_t)
+        blob = hs._hip_attention_cache
+        xin = xd.clone()
+        ops.triattn_forward(xin, md, blob, 4, True, residual=xin, out=xin)
+        assert_close(xin, x.float() + want, "triattn residual in place", rel_fro=5e-3)
