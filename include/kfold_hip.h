@@ -102,6 +102,83 @@ int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, co
                         void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                         int H, int ending, float eps, int io_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Transition (Algorithm 11, SwiGLU).  Replaces the torch modules
+ * model/layers/folding/transition.py:48-68 + model/primitives/activation.py:27-29, which the
+ * reference runs unfused on every backend.  C = 128 with expansion 2 or 4 (the pair track)
+ * runs as one fused kernel and needs no workspace; other channel counts (multiples of 128 up
+ * to 2048: the token track) run as LayerNorm + two MFMA linears through the workspace.
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_transition_packed_bytes(int C, int expansion);
+
+/* ln_* [C]; swiglu_w [2*C*expansion, C] (`swiglu.linear`); out_w [C, C*expansion] (`linear_out`). */
+int kfh_transition_pack(const void* ln_w, const void* ln_b, const void* swiglu_w, const void* out_w,
+                        int w_dtype, int C, int expansion, void* blob, void* stream);
+
+size_t kfh_transition_workspace_bytes(long long rows, int C, int expansion);
+
+/* out[r,:] = ((residual ? residual[r,:] : 0) + Transition(x[r,:])) * (mask ? mask[r] != 0 : 1)
+ * for r < rows; x, out, residual: [rows, C].  `out` may alias `x` and `residual`.  `mask`
+ * (C = 128 only, else NULL) is the final `z * pair_mask` of modules/apo_module.py:172. */
+int kfh_transition_forward(const void* x, const void* blob, const void* residual, const uint8_t* mask,
+                           void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
+                           int expansion, float eps, int io_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Pair bias of the token-track attention, as fp32 "bias tiles": the layout the attention
+ * kernel reads, [batch][head][query block of 32][key block of 32][4 KiB tile], values
+ * pre-multiplied by log2(e).
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_bias_tiles_bytes(int nbatch, int H, int L);
+
+/* tiles <- dense pair bias [nbatch, H, L, L] (io_dtype), the `pair_bias` argument of
+ * model/primitives/attention.py:28-37. */
+int kfh_bias_tiles_from_dense(const void* dense, int io_dtype, void* tiles, int nbatch, int H, int L,
+                              void* stream);
+
+/* tiles <- linear_pair_bias(layernorm_z(z)) moved to [B, H, N, N]
+ * (model/modules/confidence_head.py:162-163) in one pass over z [B, N, N, C]; w is [H, C]. */
+size_t kfh_pair_bias_packed_bytes(int C, int H);
+int kfh_pair_bias_pack(const void* ln_w, const void* ln_b, const void* w, int w_dtype, int C, int H,
+                       void* blob, void* stream);
+int kfh_pair_bias_project(const void* z, const void* blob, void* tiles, int B, int N, int C, int H,
+                          float eps, int io_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------
+ * Self attention with pair bias (Algorithm 24).  Replaces
+ * kernels/triton/attention_pair_bias/dispatch.py:370 `triton_attention_pair_bias` as called
+ * from model/primitives/attention.py:62-66, and with apply_norm != 0 the whole
+ * `SelfAttentionPairBias.forward` (model/layers/folding/attention_pair_bias.py:114-158);
+ * math of the torch path at attention.py:75-94, :239-271, :122-168.
+ * C = channel_a, H heads of C/H (<= 64) channels, Cs = conditioning channels (0 = none).
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_apb_packed_bytes(int C, int H, int Cs);
+
+/* q_w,k_w,v_w,g_w,o_w [C, C]; q_b [C] or NULL (`linear_q.bias`); unconditioned: ln_w, ln_b [C]
+ * (`layernorm_a`); conditioned (Cs > 0): adaln_s_w [Cs] (`adaln_a.layernorm_s.weight`),
+ * adaln_g_w [C, Cs] + adaln_g_b [C] (`adaln_a.linear_g`), adaln_bias_w [C, Cs]
+ * (`adaln_a.linear_bias`), ada_out_w [C, Cs] + ada_out_b [C] (`linear_ada_out`). */
+int kfh_apb_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* q_b, const void* k_w,
+                 const void* v_w, const void* g_w, const void* o_w, const void* adaln_s_w,
+                 const void* adaln_g_w, const void* adaln_g_b, const void* adaln_bias_w,
+                 const void* ada_out_w, const void* ada_out_b, int w_dtype, int C, int H, int Cs,
+                 void* blob, void* stream);
+
+size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs);
+
+/* a, out, residual: [S, L, C]; s_cond: [S or 1, L, Cs]; bias_tiles: [S or 1] batches of tiles;
+ * mask: [S or 1, L] bytes (valid keys); the *_per_sample flags say which of the two.
+ * apply_norm = 0: `a` is already normalised (the functional entry, attention.py:28) and no
+ * conditioning gate is applied; apply_norm != 0: LayerNorm (Cs = 0) or AdaLN + the
+ * sigmoid(linear_ada_out(s)) output gate (Cs > 0) are applied as the module does.
+ * out = (residual or 0) + result; `residual` may alias `out`, `out` must not alias `a`
+ * unless residual == a.  Fully masked key sets give uniform attention (finite -1e9). */
+int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, const uint8_t* mask,
+                    const void* blob, const void* residual, void* out, void* workspace,
+                    size_t workspace_bytes, int S, int L, int C, int H, int Cs, int apply_norm,
+                    int bias_per_sample, int mask_per_sample, int s_per_sample, float eps,
+                    int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

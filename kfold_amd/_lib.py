@@ -7,7 +7,7 @@ The library is loaded on first use.  There is no fallback: if it has not been bu
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_size_t, c_void_p
 from pathlib import Path
 
 LIB_PATH = Path(__file__).resolve().parent / "libkfold_hip.so"
@@ -30,6 +30,21 @@ SIGNATURES: dict[str, tuple] = {
     "kfh_triattn_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "kfh_triattn_forward": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                     c_int, c_float, c_int, _P]),
+    "kfh_transition_packed_bytes": (c_size_t, [c_int, c_int]),
+    "kfh_transition_pack": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, _P, _P]),
+    "kfh_transition_workspace_bytes": (c_size_t, [c_longlong, c_int, c_int]),
+    "kfh_transition_forward": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_longlong, c_int, c_int,
+                                       c_float, c_int, _P]),
+    "kfh_bias_tiles_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "kfh_bias_tiles_from_dense": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P]),
+    "kfh_pair_bias_packed_bytes": (c_size_t, [c_int, c_int]),
+    "kfh_pair_bias_pack": (c_int, [_P, _P, _P, c_int, c_int, c_int, _P, _P]),
+    "kfh_pair_bias_project": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+    "kfh_apb_packed_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "kfh_apb_pack": (c_int, [_P] * 14 + [c_int, c_int, c_int, c_int, _P, _P]),
+    "kfh_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "kfh_apb_forward": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
+                                c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
 }
 
 _lib = None

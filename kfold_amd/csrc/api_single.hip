@@ -1,0 +1,379 @@
+// C ABI, single (token) track: pair bias, pair-bias attention, generic transition.
+#include "../../include/kfold_hip.h"
+
+#include <cmath>
+
+#include "api_util.hpp"
+#include "kernels.hpp"
+
+using namespace kfh;
+
+namespace {
+
+// ---- blob / workspace layouts -------------------------------------------------------------
+struct ApbLayout {
+    int C, H, Dh, PB, Cs, kq, nhb, ko;
+    size_t wq, wk, wv, wg, wo, w_adag, w_adab, w_adaout, f_bq, f_ln_g, f_ln_b, f_lns_g, f_adag_b,
+        f_adaout_b, total;
+    bool ok;
+    ApbLayout(int C_, int H_, int Cs_) : C(C_), H(H_), Cs(Cs_) {
+        ok = C > 0 && H > 0 && C % H == 0 && C % 128 == 0 && C <= 2048 && (Cs == 0 || (Cs % 128 == 0 && Cs <= 2048));
+        if (!ok) { total = 0; return; }
+        Dh = C / H;
+        PB = (Dh + 31) / 32;
+        ok = PB <= 2;
+        if (!ok) { total = 0; return; }
+        kq = C / 16;
+        nhb = H * PB;
+        ko = nhb * 2;
+        size_t off = 0;
+        auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
+        const size_t wh = (size_t)nhb * kq * 1024;
+        wq = take(wh); wk = take(wh); wv = take(wh); wg = take(wh);
+        wo = take((size_t)(C / 32) * ko * 1024);
+        const size_t wa = Cs ? (size_t)(C / 32) * (Cs / 16) * 1024 : 0;
+        w_adag = take(wa); w_adab = take(wa); w_adaout = take(wa);
+        f_bq = take(C * 4); f_ln_g = take(C * 4); f_ln_b = take(C * 4);
+        f_lns_g = take(Cs * 4); f_adag_b = take(C * 4); f_adaout_b = take(C * 4);
+        total = off;
+    }
+};
+
+struct ApbWs {
+    size_t xn, an, sn, sraw, gate_out, qf, kf, vf, gf, of, codes, total;
+    int nb;
+    ApbWs(const ApbLayout& l, int S, int L) {
+        nb = (L + 31) / 32;
+        size_t off = 0;
+        auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
+        const size_t rows = (size_t)S * L;
+        xn = take(rows * l.C * 2);
+        an = take(l.Cs ? rows * l.C * 2 : 0);
+        sn = take(l.Cs ? rows * l.Cs * 2 : 0);
+        sraw = take(l.Cs ? rows * l.Cs * 2 : 0);
+        gate_out = take(l.Cs ? rows * l.C * 2 : 0);
+        const size_t frag = (size_t)S * l.H * nb * l.PB * 2048;
+        qf = take(frag); kf = take(frag); vf = take(frag); gf = take(frag); of = take(frag);
+        codes = take((size_t)S * nb * 32);
+        total = off;
+    }
+};
+
+struct GtLayout {   // generic transition
+    size_t wu, wv, wo, f_ln, total;
+    int hid;
+    GtLayout(int C, int E) {
+        hid = C * E;
+        size_t off = 0;
+        auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
+        wu = take((size_t)(hid / 32) * (C / 16) * 1024);
+        wv = take((size_t)(hid / 32) * (C / 16) * 1024);
+        wo = take((size_t)(C / 32) * (hid / 16) * 1024);
+        f_ln = take(2 * C * 4);
+        total = off;
+    }
+};
+
+LinearArgs plain(const void* A, long long lda, long long M, int K, const void* W, int Nout) {
+    LinearArgs p{};
+    p.A = A; p.lda = lda; p.rows_a = 1; p.L = (int)M; p.nb = (int)((M + 31) / 32); p.K = K;
+    p.W = W; p.nblk = (Nout + 31) / 32; p.Nout = Nout; p.bias_scale = 1.f;
+    p.H = 1; p.PB = 1; p.Dh = 32;
+    return p;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ------------------------------------------------------------------------------------------
+// pair bias tiles
+// ------------------------------------------------------------------------------------------
+size_t kfh_bias_tiles_bytes(int nbatch, int H, int L) {
+    if (nbatch <= 0 || H <= 0 || L <= 0) return 0;
+    const size_t nb = (L + 31) / 32;
+    return align_up((size_t)nbatch * H * nb * nb * 4096);
+}
+
+int kfh_bias_tiles_from_dense(const void* dense, int io_dtype, void* tiles, int nbatch, int H, int L,
+                              void* stream) {
+    if (!dense || !tiles || nbatch <= 0 || H <= 0 || L <= 0)
+        return fail(KFH_EINVAL, "bias_tiles_from_dense: bad argument");
+    if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "bias_tiles_from_dense: bad io_dtype %d", io_dtype);
+    launch_bias_tiles(dense, io_dtype, static_cast<float*>(tiles), nbatch, H, L, (L + 31) / 32,
+                      static_cast<hipStream_t>(stream));
+    return check_launch("bias_tiles_from_dense");
+}
+
+size_t kfh_pair_bias_packed_bytes(int C, int H) {
+    return (C == kC && H >= 1 && H <= 32) ? align_up(kPbBlobBytes) : 0;
+}
+
+int kfh_pair_bias_pack(const void* ln_w, const void* ln_b, const void* w, int w_dtype, int C, int H,
+                       void* blob, void* stream_) {
+    if (C != kC || H < 1 || H > 32)
+        return fail(KFH_EUNSUPPORTED, "pair_bias_pack: C=%d H=%d, built for C=128, H<=32", C, H);
+    if (!dtype_ok(w_dtype) || !w || !blob) return fail(KFH_EINVAL, "pair_bias_pack: bad argument");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* b = static_cast<char*>(blob);
+    launch_pack_blocks(w, w_dtype, H, C, C, 0, 1, ROW_NATURAL, K_NATURAL, kLog2e, b, stream);
+    float* ln = reinterpret_cast<float*>(b + kBlockBytes);
+    launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);
+    launch_copy_f32(ln_b, w_dtype, ln + C, C, 0.f, stream);
+    return check_launch("pair_bias_pack");
+}
+
+int kfh_pair_bias_project(const void* z, const void* blob, void* tiles, int B, int N, int C, int H,
+                          float eps, int io_dtype, void* stream_) {
+    if (C != kC || H < 1 || H > 32)
+        return fail(KFH_EUNSUPPORTED, "pair_bias_project: C=%d H=%d, built for C=128, H<=32", C, H);
+    if (!z || !blob || !tiles || B <= 0 || N <= 0 || !dtype_ok(io_dtype))
+        return fail(KFH_EINVAL, "pair_bias_project: bad argument");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const size_t nb = (N + 31) / 32, esz = io_dtype == KFH_F32 ? 4 : 2;
+    for (int b = 0; b < B; ++b) {
+        float* t = static_cast<float*>(tiles) + (size_t)b * H * nb * nb * 1024;
+        if (N % 32) {   // queries beyond N in the last query block: keep their tiles finite
+            for (int h = 0; h < H; ++h)
+                launch_fill_zero(t + (((size_t)h * nb + (nb - 1)) * nb) * 1024, nb * 4096, stream);
+        }
+        launch_pair_bias(static_cast<const char*>(z) + (size_t)b * N * N * C * esz, io_dtype,
+                         static_cast<const char*>(blob), t, N, H, eps, stream);
+    }
+    return check_launch("pair_bias_project");
+}
+
+// ------------------------------------------------------------------------------------------
+// pair-bias attention
+// ------------------------------------------------------------------------------------------
+size_t kfh_apb_packed_bytes(int C, int H, int Cs) { return ApbLayout(C, H, Cs).total; }
+
+int kfh_apb_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* q_b, const void* k_w,
+                 const void* v_w, const void* g_w, const void* o_w, const void* adaln_s_w,
+                 const void* adaln_g_w, const void* adaln_g_b, const void* adaln_bias_w,
+                 const void* ada_out_w, const void* ada_out_b, int w_dtype, int C, int H, int Cs,
+                 void* blob, void* stream_) {
+    const ApbLayout l(C, H, Cs);
+    if (!l.ok) return fail(KFH_EUNSUPPORTED, "apb_pack: C=%d H=%d Cs=%d not supported (C,Cs multiples of 128 up to 2048, head dim <= 64)", C, H, Cs);
+    if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "apb_pack: bad w_dtype %d", w_dtype);
+    if (!q_w || !k_w || !v_w || !g_w || !o_w || !blob) return fail(KFH_EINVAL, "apb_pack: null pointer");
+    if (Cs && (!adaln_g_w || !adaln_bias_w || !ada_out_w))
+        return fail(KFH_EINVAL, "apb_pack: conditioned module needs the AdaLN / ada_out weights");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* b = static_cast<char*>(blob);
+    const float qscale = kLog2e / sqrtf((float)l.Dh);
+    const size_t blk = (size_t)l.kq * 1024;
+    for (int h = 0; h < H; ++h)
+        for (int pp = 0; pp < l.PB; ++pp) {
+            const int rows = l.Dh - 32 * pp < 32 ? l.Dh - 32 * pp : 32;
+            const int row0 = h * l.Dh + 32 * pp;
+            const size_t o = (size_t)(h * l.PB + pp) * blk;
+            launch_pack_blocks(q_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, qscale, b + l.wq + o, stream);
+            launch_pack_blocks(k_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wk + o, stream);
+            launch_pack_blocks(v_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wv + o, stream);
+            launch_pack_blocks(g_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wg + o, stream);
+        }
+    launch_pack_blocks(o_w, w_dtype, C, l.ko * 16, C, 0, C / 32, ROW_NATURAL, K_ACC_HEADPAD, 1.f, b + l.wo,
+                       stream, l.Dh | ((2 * l.PB) << 16));
+    launch_copy_f32(q_b, w_dtype, reinterpret_cast<float*>(b + l.f_bq), C, 0.f, stream);
+    launch_copy_f32(ln_w, w_dtype, reinterpret_cast<float*>(b + l.f_ln_g), C, 1.f, stream);
+    launch_copy_f32(ln_b, w_dtype, reinterpret_cast<float*>(b + l.f_ln_b), C, 0.f, stream);
+    if (Cs) {
+        launch_pack_blocks(adaln_g_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adag, stream);
+        launch_pack_blocks(adaln_bias_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adab, stream);
+        launch_pack_blocks(ada_out_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adaout, stream);
+        launch_copy_f32(adaln_s_w, w_dtype, reinterpret_cast<float*>(b + l.f_lns_g), Cs, 1.f, stream);
+        launch_copy_f32(adaln_g_b, w_dtype, reinterpret_cast<float*>(b + l.f_adag_b), C, 0.f, stream);
+        launch_copy_f32(ada_out_b, w_dtype, reinterpret_cast<float*>(b + l.f_adaout_b), C, 0.f, stream);
+    }
+    return check_launch("apb_pack");
+}
+
+size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs) {
+    const ApbLayout l(C, H, Cs);
+    if (!l.ok || S <= 0 || L <= 0 || L > 8192) return 0;
+    return ApbWs(l, S, L).total;
+}
+
+int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, const uint8_t* mask,
+                    const void* blob, const void* residual, void* out, void* workspace,
+                    size_t workspace_bytes, int S, int L, int C, int H, int Cs, int apply_norm,
+                    int bias_per_sample, int mask_per_sample, int s_per_sample, float eps,
+                    int io_dtype, void* stream_) {
+    const ApbLayout l(C, H, Cs);
+    if (!l.ok) return fail(KFH_EUNSUPPORTED, "apb_forward: C=%d H=%d Cs=%d not supported", C, H, Cs);
+    if (S <= 0 || L <= 0) return fail(KFH_EINVAL, "apb_forward: bad shape S=%d L=%d", S, L);
+    if (L > 8192) return fail(KFH_EUNSUPPORTED, "apb_forward: L=%d > 8192", L);
+    if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "apb_forward: bad io_dtype %d", io_dtype);
+    if (!a || !bias_tiles || !mask || !blob || !out || !workspace)
+        return fail(KFH_EINVAL, "apb_forward: null pointer argument");
+    const bool cond = Cs > 0 && apply_norm;
+    if (cond && !s_cond) return fail(KFH_EINVAL, "apb_forward: conditioned module needs s_cond");
+    const ApbWs w(l, S, L);
+    if (workspace_bytes < w.total)
+        return fail(KFH_EINVAL, "apb_forward: workspace %zu < %zu bytes", workspace_bytes, w.total);
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* b = static_cast<const char*>(blob);
+    char* ws = static_cast<char*>(workspace);
+    const long long rows = (long long)S * L;
+    auto f32p = [&](size_t off) { return reinterpret_cast<const float*>(b + off); };
+    uint16_t* xn = reinterpret_cast<uint16_t*>(ws + w.xn);
+
+    // 1. normalised input rows (bf16)
+    if (!apply_norm) {
+        launch_rows_norm(a, io_dtype, nullptr, nullptr, xn, rows, C, 0, eps, stream);
+    } else if (!Cs) {
+        launch_rows_norm(a, io_dtype, f32p(l.f_ln_g), f32p(l.f_ln_b), xn, rows, C, 1, eps, stream);
+    } else {
+        // AdaLN: sigmoid(W_g LN_s(s) + b_g) * LN(a) + W_b LN_s(s)
+        const long long srows = s_per_sample ? rows : L;
+        uint16_t* an = reinterpret_cast<uint16_t*>(ws + w.an);
+        uint16_t* sn = reinterpret_cast<uint16_t*>(ws + w.sn);
+        uint16_t* sraw = reinterpret_cast<uint16_t*>(ws + w.sraw);
+        launch_rows_norm(a, io_dtype, nullptr, nullptr, an, rows, C, 1, eps, stream);
+        launch_rows_norm(s_cond, io_dtype, f32p(l.f_lns_g), nullptr, sn, srows, Cs, 1, eps, stream);
+        launch_rows_norm(s_cond, io_dtype, nullptr, nullptr, sraw, srows, Cs, 0, eps, stream);
+        LinearArgs p = plain(sn, Cs, L, Cs, b + l.w_adag, C);
+        p.rows_a = S; p.a_shared = !s_per_sample;
+        p.W2 = b + l.w_adab; p.bias = f32p(l.f_adag_b);
+        p.aux = an; p.aux_dtype = KFH_BF16; p.ld_aux = C;
+        p.out = xn; p.out_dtype = KFH_BF16; p.ldo = C; p.epi = EPI_ADALN;
+        launch_linear(p, stream);
+        // output gate sigmoid(W_ada s + b_ada) on the raw conditioning
+        LinearArgs g = plain(sraw, Cs, srows, Cs, b + l.w_adaout, C);
+        g.bias = f32p(l.f_adaout_b);
+        g.out = ws + w.gate_out; g.out_dtype = KFH_BF16; g.ldo = C; g.epi = EPI_SIGMOID;
+        launch_linear(g, stream);
+    }
+
+    // 2. q (with bias, pre-scaled), k, gate, v projections into fragment order
+    {
+        LinearArgs p = plain(xn, C, L, C, nullptr, C);
+        p.rows_a = S; p.nblk = l.nhb; p.H = H; p.PB = l.PB; p.Dh = l.Dh;
+        p.epi = EPI_FRAG_CH;
+        p.W = b + l.wq; p.bias = f32p(l.f_bq); p.bias_scale = kLog2e / sqrtf((float)l.Dh);
+        p.out = ws + w.qf;
+        launch_linear(p, stream);
+        p.bias = nullptr;
+        p.W = b + l.wk; p.out = ws + w.kf;
+        launch_linear(p, stream);
+        p.W = b + l.wg; p.out = ws + w.gf; p.sigmoid = 1;
+        launch_linear(p, stream);
+        p.sigmoid = 0; p.epi = EPI_FRAG_POS;
+        p.W = b + l.wv; p.out = ws + w.vf;
+        launch_linear(p, stream);
+    }
+
+    // 3. key codes, attention
+    uint8_t* codes = reinterpret_cast<uint8_t*>(ws + w.codes);
+    launch_key_codes(mask, codes, S, L, w.nb * 32, mask_per_sample ? L : 0, stream);
+    FlashArgs fa{};
+    fa.qf = ws + w.qf; fa.kf = ws + w.kf; fa.vf = ws + w.vf; fa.gf = ws + w.gf; fa.of = ws + w.of;
+    fa.biasf = bias_tiles; fa.codes = codes;
+    fa.nrows = S; fa.nb = w.nb; fa.H = H; fa.bias_per_row = bias_per_sample ? 1 : 0;
+    if (launch_flash(fa, 32 * l.PB, stream) != 0) return fail(KFH_EUNSUPPORTED, "apb_forward: attention shape");
+
+    // 4. output projection (+ conditioning gate, + residual)
+    {
+        LinearArgs p{};
+        p.A = ws + w.of; p.a_frag = 1; p.rows_a = S; p.L = L; p.nb = w.nb; p.K = l.ko * 16;
+        p.W = b + l.wo; p.nblk = C / 32; p.Nout = C; p.bias_scale = 1.f;
+        p.H = H; p.PB = l.PB; p.Dh = l.Dh;
+        p.epi = EPI_RESID;
+        if (cond) { p.gate = reinterpret_cast<const uint16_t*>(ws + w.gate_out); p.ld_gate = C; p.gate_shared = !s_per_sample; }
+        if (residual) { p.aux = residual; p.aux_dtype = io_dtype; p.ld_aux = C; }
+        p.out = out; p.out_dtype = io_dtype; p.ldo = C;
+        launch_linear(p, stream);
+    }
+    return check_launch("apb_forward");
+}
+
+// ------------------------------------------------------------------------------------------
+// transition for any channel count (token track); C = 128 uses the fused pair kernel
+// ------------------------------------------------------------------------------------------
+size_t kfh_transition_packed_bytes(int C, int expansion) {
+    if (C == kC && (expansion == 2 || expansion == 4)) return align_up(transition_blob_bytes(expansion));
+    if (C <= 0 || C % 128 || C > 2048 || expansion < 1 || expansion > 8) return 0;
+    return GtLayout(C, expansion).total;
+}
+
+int kfh_transition_pack(const void* ln_w, const void* ln_b, const void* swiglu_w, const void* out_w,
+                        int w_dtype, int C, int expansion, void* blob, void* stream_) {
+    if (kfh_transition_packed_bytes(C, expansion) == 0)
+        return fail(KFH_EUNSUPPORTED, "transition_pack: C=%d E=%d not supported", C, expansion);
+    if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "transition_pack: bad w_dtype %d", w_dtype);
+    if (!swiglu_w || !out_w || !blob) return fail(KFH_EINVAL, "transition_pack: null pointer");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    char* b = static_cast<char*>(blob);
+    const int hid = C * expansion;
+    const size_t wsz = w_dtype == KFH_F32 ? 4 : 2;
+    if (C == kC && (expansion == 2 || expansion == 4)) {
+        const int nstep = hid / 32;
+        for (int s = 0; s < nstep; ++s) {
+            char* step = b + (size_t)s * 3 * kBlockBytes;
+            launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, 32 * s, 1, ROW_NATURAL, K_NATURAL, 1.f, step, stream);
+            launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, hid + 32 * s, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                               step + kBlockBytes, stream);
+            // W_out[:, 32s .. 32s+31]: a 32-wide column slice of the [C, hid] matrix
+            launch_pack_blocks(static_cast<const char*>(out_w) + (size_t)32 * s * wsz, w_dtype, C, 32, hid,
+                               0, 4, ROW_INTERLEAVE4, K_ACC, 1.f, step + 2 * kBlockBytes, stream);
+        }
+        float* ln = reinterpret_cast<float*>(b + (size_t)nstep * 3 * kBlockBytes);
+        launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);
+        launch_copy_f32(ln_b, w_dtype, ln + C, C, 0.f, stream);
+    } else {
+        const GtLayout l(C, expansion);
+        launch_pack_blocks(swiglu_w, w_dtype, hid, C, C, 0, hid / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.wu, stream);
+        launch_pack_blocks(swiglu_w, w_dtype, hid, C, C, hid, hid / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.wv, stream);
+        launch_pack_blocks(out_w, w_dtype, C, hid, hid, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.wo, stream);
+        float* ln = reinterpret_cast<float*>(b + l.f_ln);
+        launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);
+        launch_copy_f32(ln_b, w_dtype, ln + C, C, 0.f, stream);
+    }
+    return check_launch("transition_pack");
+}
+
+size_t kfh_transition_workspace_bytes(long long rows, int C, int expansion) {
+    if (C == kC && (expansion == 2 || expansion == 4)) return 0;
+    if (rows <= 0 || kfh_transition_packed_bytes(C, expansion) == 0) return 0;
+    return align_up((size_t)rows * C * 2) + align_up((size_t)rows * C * expansion * 2);
+}
+
+int kfh_transition_forward(const void* x, const void* blob, const void* residual, const uint8_t* mask,
+                           void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
+                           int expansion, float eps, int io_dtype, void* stream_) {
+    if (kfh_transition_packed_bytes(C, expansion) == 0)
+        return fail(KFH_EUNSUPPORTED, "transition_forward: C=%d E=%d not supported", C, expansion);
+    if (rows < 0) return fail(KFH_EINVAL, "transition_forward: rows=%lld", rows);
+    if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "transition_forward: bad io_dtype %d", io_dtype);
+    if (!x || !blob || !out) return fail(KFH_EINVAL, "transition_forward: null pointer argument");
+    if (rows == 0) return KFH_OK;
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    const char* b = static_cast<const char*>(blob);
+    if (C == kC && (expansion == 2 || expansion == 4)) {
+        launch_pair_transition(x, io_dtype, b, expansion, residual, mask, out, rows, eps, stream);
+        return check_launch("transition_forward");
+    }
+    if (mask) return fail(KFH_EUNSUPPORTED, "transition_forward: the row mask is built for C=128 only");
+    if (rows > 0x7fffffffLL) return fail(KFH_EUNSUPPORTED, "transition_forward: too many rows");
+    const size_t need = kfh_transition_workspace_bytes(rows, C, expansion);
+    if (!workspace || workspace_bytes < need)
+        return fail(KFH_EINVAL, "transition_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+    const GtLayout l(C, expansion);
+    char* ws = static_cast<char*>(workspace);
+    uint16_t* xn = reinterpret_cast<uint16_t*>(ws);
+    uint16_t* hid = reinterpret_cast<uint16_t*>(ws + align_up((size_t)rows * C * 2));
+    const float* ln = reinterpret_cast<const float*>(b + l.f_ln);
+    launch_rows_norm(x, io_dtype, ln, ln + C, xn, rows, C, 1, eps, stream);
+    LinearArgs p = plain(xn, C, rows, C, b + l.wu, l.hid);
+    p.W2 = b + l.wv; p.out = hid; p.out_dtype = KFH_BF16; p.ldo = l.hid; p.epi = EPI_SWIGLU;
+    launch_linear(p, stream);
+    LinearArgs q = plain(hid, l.hid, rows, l.hid, b + l.wo, C);
+    q.epi = EPI_RESID;
+    if (residual) { q.aux = residual; q.aux_dtype = io_dtype; q.ld_aux = C; }
+    q.out = out; q.out_dtype = io_dtype; q.ldo = C;
+    launch_linear(q, stream);
+    return check_launch("transition_forward");
+}
+
+}  // extern "C"

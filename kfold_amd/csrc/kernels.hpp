@@ -6,13 +6,14 @@ namespace kfh {
 
 // ---- weight packing (pack.hip) ----------------------------------------------------------
 enum : int { ROW_NATURAL = 0, ROW_INTERLEAVE2 = 1, ROW_INTERLEAVE4 = 2 };
-enum : int { K_NATURAL = 0, K_ACC = 1, K_HALF = 2 };
+enum : int { K_NATURAL = 0, K_ACC = 1, K_HALF = 2, K_ACC_HEADPAD = 3 };
 
 constexpr size_t kBlockBytes = 32 * kC * 2;   // one packed 32-row x 128-channel block = 8 KiB
 
+// K: number of k-slots (padded contraction length); ld: row pitch of src in elements
 void launch_pack_blocks(const void* src, int wdtype, int src_rows, int K, int ld, int row0,
                         int nblk, int row_mode, int k_mode, float scale, void* dst,
-                        hipStream_t stream);
+                        hipStream_t stream, int kparam = 0);
 void launch_copy_f32(const void* src, int wdtype, float* dst, int n, float fill,
                      hipStream_t stream);
 
@@ -58,9 +59,62 @@ struct TriattnWorkspace {
     uint8_t* codes;                  // N * nb * 32 key codes
 };
 
+// ---- attention core (flash.hip) --------------------------------------------------------------
+struct FlashArgs {
+    const void *qf, *kf, *vf, *gf;   // fragment-order operands
+    void* of;                         // gated output fragments
+    const void* biasf;                // fp32 bias tiles
+    const uint8_t* codes;             // [nrows][nb*32] key codes
+    int nrows, nb, H;
+    int bias_per_row;                 // 0: one bias for all rows, 1: bias batch index = row
+    int qgroups, nchunks;             // filled in by launch_flash
+};
+int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
+
 void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream);
 void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
                     float eps, hipStream_t stream);
+
+// ---- pair transition (transition.hip) ----------------------------------------------------
+// Packed blob (C = 128, expansion E): 4E steps x 24 KiB { u block, v block, W_out slice of the
+// step's 32 hidden channels as 4 blocks x 2 k-steps (ROW_INTERLEAVE4, K_ACC) }, then fp32 LN
+// gamma, beta.
+inline size_t transition_blob_bytes(int E) { return (size_t)4 * E * 3 * kBlockBytes + 2 * kC * sizeof(float); }
+int launch_pair_transition(const void* x, int io_dtype, const char* blob, int expansion,
+                           const void* residual, const uint8_t* mask, void* out, long long M,
+                           float eps, hipStream_t stream);
+
+// ---- pair bias projection (pairbias.hip): blob = one packed block (heads as rows, scaled by
+// log2 e) followed by fp32 LN gamma, beta
+constexpr size_t kPbBlobBytes = kBlockBytes + 2 * kC * sizeof(float);
+void launch_pair_bias(const void* z, int io_dtype, const char* blob, float* tiles, int N, int H,
+                      float eps, hipStream_t stream);
+
+// ---- single-track helpers (rows.hip, linear.hip) -------------------------------------------
+int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
+                     long long M, int C, int normalize, float eps, hipStream_t stream);
+void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
+                      long long mask_stride, hipStream_t stream);
+void launch_bias_tiles(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
+                       hipStream_t stream);
+
+enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS };
+
+// Rows are addressed as (a, position): a < rows_a, position < L, global row = a * L + position,
+// position blocks of 32 (nb = ceil(L / 32)).  Plain [M, K] problems use rows_a = 1, L = M.
+struct LinearArgs {
+    const void* A; long long lda; int a_frag;    // row-major bf16 [rows][lda] or fragment order
+    int a_shared, aux_shared, gate_shared;       // operand has one `a` slice shared by all rows_a
+    int rows_a, L, nb, K;                        // K: contraction length in the packed weight
+    const void* W; const void* W2; int nblk;     // packed blocks [nblk][K/16][64 lanes][8]
+    const float* bias; float bias_scale; int sigmoid;
+    const void* aux; int aux_dtype; long long ld_aux;
+    const uint16_t* gate; long long ld_gate;
+    void* out; int out_dtype; long long ldo; int Nout;
+    int epi;
+    int H, PB, Dh;                               // heads, 32-blocks per padded head, real head dim
+};
+int launch_linear(const LinearArgs& p, hipStream_t stream);
 
 }  // namespace kfh

@@ -19,19 +19,26 @@ __device__ __forceinline__ int pack_row(int mode, int b, int col) {
     }
 }
 
-__device__ __forceinline__ int pack_k(int mode, int K, int ks, int half, int e) {
+// source column of k-slot (ks, half, e), or -1 for a zero (padding) slot
+__device__ __forceinline__ int pack_k(int mode, int K, int ks, int half, int e, int kparam) {
     switch (mode) {
         case K_NATURAL: return 16 * ks + 8 * half + e;
         case K_ACC: return 16 * ks + 8 * (e >> 2) + 4 * half + (e & 3);
         case K_HALF: return (K >> 1) * half + 8 * ks + e;
+        case K_ACC_HEADPAD: {
+            // k-steps are grouped per head: kparam = (real head dim) | (k-steps per padded head) << 16
+            const int dh = kparam & 0xffff, dks = kparam >> 16;
+            const int h = ks / dks, d = 16 * (ks % dks) + 8 * (e >> 2) + 4 * half + (e & 3);
+            return d < dh ? h * dh + d : -1;
+        }
         default: return 16 * ks + 8 * half + e;
     }
 }
 
 template <int WT>
 __global__ void pack_blocks_kernel(const void* __restrict__ src, int src_rows, int K, int ld,
-                                   int row0, int nblk, int row_mode, int k_mode, float scale,
-                                   uint16_t* __restrict__ dst) {
+                                   int row0, int nblk, int row_mode, int k_mode, int kparam,
+                                   float scale, uint16_t* __restrict__ dst) {
     const int ksteps = K / 16;
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;      // (block, ks, lane)
     if (idx >= nblk * ksteps * 64) return;
@@ -46,9 +53,9 @@ __global__ void pack_blocks_kernel(const void* __restrict__ src, int src_rows, i
         float v[2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int k = pack_k(k_mode, K, ks, half, e + u);
+            const int k = pack_k(k_mode, K, ks, half, e + u, kparam);
             float x = 0.f;
-            if (r < src_rows) {
+            if (r < src_rows && k >= 0) {
                 const size_t off = (size_t)(row0 + r) * ld + k;
                 if constexpr (WT == KFH_F32) x = static_cast<const float*>(src)[off];
                 else x = bf16_lo(static_cast<const uint16_t*>(src)[off]);
@@ -90,16 +97,16 @@ void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream) {
 
 void launch_pack_blocks(const void* src, int wdtype, int src_rows, int K, int ld, int row0,
                         int nblk, int row_mode, int k_mode, float scale, void* dst,
-                        hipStream_t stream) {
+                        hipStream_t stream, int kparam) {
     const int total = nblk * (K / 16) * 64;
     const int threads = 256, blocks = (total + threads - 1) / threads;
     if (wdtype == KFH_F32)
         hipLaunchKernelGGL(pack_blocks_kernel<KFH_F32>, dim3(blocks), dim3(threads), 0, stream, src,
-                           src_rows, K, ld, row0, nblk, row_mode, k_mode, scale,
+                           src_rows, K, ld, row0, nblk, row_mode, k_mode, kparam, scale,
                            static_cast<uint16_t*>(dst));
     else
         hipLaunchKernelGGL(pack_blocks_kernel<KFH_BF16>, dim3(blocks), dim3(threads), 0, stream, src,
-                           src_rows, K, ld, row0, nblk, row_mode, k_mode, scale,
+                           src_rows, K, ld, row0, nblk, row_mode, k_mode, kparam, scale,
                            static_cast<uint16_t*>(dst));
 }
 

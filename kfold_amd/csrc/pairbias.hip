@@ -1,0 +1,65 @@
+// Pair bias of the single-track attention:  bias[h, q, k] = (W LN(z[q, k]))[h]
+// (reference: model/modules/confidence_head.py:162-163, `linear_pair_bias(layernorm_z(z))`
+// moved to [B, H, L, L]).  One pass over z, HBM-bound on the z read; the result is written
+// directly as the log2(e)-scaled fp32 bias tiles the attention kernel consumes (flash.hip).
+#include "kernels.hpp"
+
+namespace kfh {
+
+template <int IO>
+__global__ __launch_bounds__(256) void pair_bias_kernel(const void* __restrict__ z,
+                                                        const char* __restrict__ blob,
+                                                        float* __restrict__ tiles, int N, int nb,
+                                                        int H, float eps) {
+    __shared__ __attribute__((aligned(16))) char smem[256 * kXS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int a = blockIdx.y, t0 = blockIdx.x * 256;      // query a, keys t0 .. t0+255
+    stage_ln_rows<IO, 256>(smem, z, reinterpret_cast<const float*>(blob + kBlockBytes), eps, tid,
+                           [&](int row) -> long long {
+                               const int b = t0 + row;
+                               return b < N ? (long long)(((size_t)a * N + b) * kC) : -1;
+                           });
+    __syncthreads();
+    const int blk0 = (t0 + wave * 64) >> 5;
+    const bf16x8* w = reinterpret_cast<const bf16x8*>(blob) + lane;
+    f32x16 acc[2];
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[pb][v] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) {
+        const bf16x8 wk = w[ks * 64];
+#pragma unroll
+        for (int pb = 0; pb < 2; ++pb)
+            acc[pb] = mfma32(wk, lds_frag(smem, wave * 64 + 32 * pb + col, ks, half), acc[pb]);
+    }
+    // accumulator rows are heads; lane col is the key inside its block
+    const int lane_q = (a & 31) + 32 * ((col >> 2) & 1);
+#pragma unroll
+    for (int pb = 0; pb < 2; ++pb) {
+        const int kblk = blk0 + pb;
+        if (kblk >= nb) continue;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int h = acc_row(v, half);
+            if (h < H) {
+                const size_t tile = ((size_t)h * nb + (a >> 5)) * nb + kblk;
+                tiles[((tile * 4 + (col >> 3)) * 64 + lane_q) * 4 + (col & 3)] = acc[pb][v];
+            }
+        }
+    }
+}
+
+void launch_pair_bias(const void* z, int io_dtype, const char* blob, float* tiles, int N, int H,
+                      float eps, hipStream_t stream) {
+    const int nb = (N + 31) / 32;
+    dim3 grid((N + 255) / 256, N), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(pair_bias_kernel<KFH_F32>, grid, block, 0, stream, z, blob, tiles, N, nb, H, eps);
+    else
+        hipLaunchKernelGGL(pair_bias_kernel<KFH_BF16>, grid, block, 0, stream, z, blob, tiles, N, nb, H, eps);
+}
+
+}  // namespace kfh

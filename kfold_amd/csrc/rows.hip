@@ -1,0 +1,126 @@
+// Small row-wise kernels of the single (token) track: LayerNorm / cast of [rows, C] tensors,
+// key-code construction and dense pair bias -> bias tiles.  These tensors are tiny next to
+// the pair representation; the kernels are plain, coalesced and wavefront-reduced.
+#include "kernels.hpp"
+
+namespace kfh {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) v += __shfl_xor(v, off);
+    return v;
+}
+
+// out[r, :] = bf16( normalize ? LN(x[r, :]) * gamma + beta : x[r, :] ), one wavefront per row.
+// gamma / beta may be null (1 / 0).  C is a multiple of 128, at most 2048.
+// (reference: model/primitives/normalization.py:61-91 — fp32 statistics, biased variance)
+template <int IO>
+__global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__ x,
+                                                        const float* __restrict__ gamma,
+                                                        const float* __restrict__ beta,
+                                                        uint16_t* __restrict__ out, long long M, int C,
+                                                        int normalize, float eps) {
+    const int lane = threadIdx.x & 63;
+    const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (r >= M) return;
+    const int npair = C / 128;
+    float a[16], b[16];
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        if (i >= npair) break;
+        const size_t e = (size_t)r * C + 128 * i + 2 * lane;
+        if constexpr (IO == KFH_BF16) {
+            const uint32_t w = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(x) + e);
+            a[i] = bf16_lo(w); b[i] = bf16_hi(w);
+        } else {
+            const f32x2 w = *reinterpret_cast<const f32x2*>(static_cast<const float*>(x) + e);
+            a[i] = w[0]; b[i] = w[1];
+        }
+        s += a[i] + b[i];
+    }
+    float mean = 0.f, rstd = 1.f;
+    if (normalize) {
+        mean = wave_sum(s) / C;
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if (i >= npair) break;
+            a[i] -= mean; b[i] -= mean; q += a[i] * a[i] + b[i] * b[i];
+        }
+        rstd = __builtin_amdgcn_rsqf(wave_sum(q) / C + eps);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        if (i >= npair) break;
+        const int c = 128 * i + 2 * lane;
+        float u = a[i] * rstd, v = b[i] * rstd;
+        if (normalize) {
+            if (gamma) { u *= gamma[c]; v *= gamma[c + 1]; }
+            if (beta) { u += beta[c]; v += beta[c + 1]; }
+        }
+        *reinterpret_cast<uint32_t*>(out + (size_t)r * C + c) = pack_bf16(u, v);
+    }
+}
+
+int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
+                     long long M, int C, int normalize, float eps, hipStream_t stream) {
+    if (C % 128 || C > 2048) return -1;
+    dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(rows_norm_kernel<KFH_F32>, grid, block, 0, stream, x, gamma, beta, out, M, C,
+                           normalize, eps);
+    else
+        hipLaunchKernelGGL(rows_norm_kernel<KFH_BF16>, grid, block, 0, stream, x, gamma, beta, out, M, C,
+                           normalize, eps);
+    return 0;
+}
+
+// codes[a][k] = k < L ? (mask[a * mask_stride + k] ? 2 : 1) : 0     for k < Lp = nb * 32
+__global__ void key_codes_kernel(const uint8_t* __restrict__ mask, uint8_t* __restrict__ codes,
+                                 int rows, int L, int Lp, long long mask_stride) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (long long)rows * Lp) return;
+    const int a = (int)(i / Lp), k = (int)(i % Lp);
+    codes[i] = k < L ? (mask[a * mask_stride + k] ? 2 : 1) : 0;
+}
+
+void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
+                      long long mask_stride, hipStream_t stream) {
+    const long long n = (long long)rows * Lp;
+    hipLaunchKernelGGL(key_codes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, mask,
+                       codes, rows, L, Lp, mask_stride);
+}
+
+// Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled fp32 tiles in accumulator order
+// [nbatch][H][qb][kb][group of 8 keys][lane = query + 32 * key-half][key % 4].
+template <int IO>
+__global__ void bias_tiles_kernel(const void* __restrict__ dense, float* __restrict__ tiles,
+                                  long long total, int H, int L, int nb) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int e = (int)(i & 3), lane = (int)((i >> 2) & 63), g = (int)((i >> 8) & 3);
+    long long t = i >> 10;
+    const int kb = (int)(t % nb); t /= nb;
+    const int qb = (int)(t % nb); t /= nb;          // t = batch * H + h
+    const int q = qb * 32 + (lane & 31), k = kb * 32 + 8 * g + 4 * (lane >> 5) + e;
+    float v = 0.f;
+    if (q < L && k < L) {
+        const size_t off = ((size_t)t * L + q) * L + k;
+        if constexpr (IO == KFH_F32) v = static_cast<const float*>(dense)[off];
+        else v = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
+    }
+    tiles[i] = v * kLog2e;
+}
+
+void launch_bias_tiles(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
+                       hipStream_t stream) {
+    const long long total = (long long)nbatch * H * nb * nb * 1024;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, H, L, nb);
+    else
+        hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, H, L, nb);
+}
+
+}  // namespace kfh

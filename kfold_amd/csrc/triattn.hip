@@ -10,7 +10,7 @@
 //     o[i,j,h]   = softmax_k(L) v[i,k,h] ;  out'[i,j] = W_o (o[i,j] * sigmoid(g[i,j]))
 //
 // triattn_proj_kernel  x' rows -> LN -> q,k,v,gate in MFMA fragment order + bias tiles + key codes
-// triattn_flash_kernel per (row, head, 32 queries): online-softmax attention over all keys
+// flash_kernel         (flash.hip) per (row, head, 32 queries): online-softmax attention
 // triattn_out_kernel   gated o fragments -> W_o -> (+ residual) -> out (transposed back)
 //
 // Fragment buffers: [row a][head h][position block of 32][k-step 0..1][lane][8 bf16], the
@@ -182,158 +182,6 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-// flash attention: wavefront = 32 queries of R rows for one head; workgroup = 4 adjacent
-// query blocks.  S^T[key][query] = K Q^T + bias is produced by the MFMA with the bias tile as
-// its C operand, so a lane owns 16 keys of one query: the row max and row sum need one
-// cross-half exchange, and exp2(S - m) rounded to bf16 is already the B operand of
-// O^T[d][query] += V^T[d][key] P^T[key][query].
-// ------------------------------------------------------------------------------------------
-template <int R>
-__global__ __launch_bounds__(256, 2) void triattn_flash_kernel(
-    const bf16x8* __restrict__ qf, const bf16x8* __restrict__ kf, const bf16x8* __restrict__ vf,
-    const bf16x8* __restrict__ gf, const f32x4* __restrict__ biasf,
-    const uint8_t* __restrict__ codes, bf16x8* __restrict__ of, int N, int nb, int qgroups,
-    int nchunks) {
-    __shared__ uint8_t cls_s[4][R][256];      // per wavefront: class of each key block per row
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int half = lane >> 5;
-
-    // chunk = (head, row set); all query groups of a chunk run on one XCD (ids are dealt
-    // round-robin over 8 XCDs), heads are the slowest index
-    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-    const int chunk = (slot / qgroups) * 8 + xcd;
-    if (chunk >= nchunks) return;
-    const int qb = (slot % qgroups) * 4 + wave;
-    const int rowsets = (N + R - 1) / R;
-    const int h = chunk / rowsets, a0 = (chunk % rowsets) * R;
-    if (qb >= nb) return;
-
-    // ---- per row: classify key blocks (0 skip, 1 mixed, 2 all valid) ------------------------
-    bool uniform_row[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int a = min(a0 + r, N - 1);
-        const uint8_t* crow = codes + (size_t)a * nb * 32;
-        bool any_valid = false;
-        for (int base = 0; base < nb; base += 64) {
-            const int blk = base + lane;
-            int nvalid = 0, nreal = 0;
-            if (blk < nb) {
-                const u32x4* p = reinterpret_cast<const u32x4*>(crow + blk * 32);
-                const u32x4 c0 = p[0], c1 = p[1];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    nvalid += __popc(c0[i] & 0x02020202u) + __popc(c1[i] & 0x02020202u);
-                    nreal += __popc(c0[i] & 0x03030303u) + __popc(c1[i] & 0x03030303u);
-                }
-            }
-            any_valid = any_valid || (__ballot(nvalid > 0) != 0ull);
-            // provisional: 2 all valid, 1 some valid, 0x80 | (real keys present) otherwise
-            if (blk < nb)
-                cls_s[wave][r][blk] = nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal > 0 ? 0x81 : 0x80));
-        }
-        uniform_row[r] = !any_valid;
-    }
-    __builtin_amdgcn_s_waitcnt(0);   // LDS writes above are read below by the same wavefront
-    __builtin_amdgcn_wave_barrier();
-
-    bf16x8 q0[R], q1[R];
-    f32x16 o[R];
-    float m[R], l[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const int a = min(a0 + r, N - 1);
-        q0[r] = qf[frag_index(a, h, qb, 0, nb, lane)];
-        q1[r] = qf[frag_index(a, h, qb, 1, nb, lane)];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) o[r][v] = 0.f;
-        m[r] = -1e30f;
-        l[r] = 0.f;
-    }
-
-    for (int kb = 0; kb < nb; ++kb) {
-        const f32x4* bt = biasf + (((size_t)h * nb + qb) * nb + kb) * 4 * 64 + lane;
-        f32x16 bias;
-        {
-            const f32x4 b0 = bt[0], b1 = bt[64], b2 = bt[128], b3 = bt[192];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { bias[e] = b0[e]; bias[4 + e] = b1[e]; bias[8 + e] = b2[e]; bias[12 + e] = b3[e]; }
-        }
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            const int a = min(a0 + r, N - 1);
-            int cls = __builtin_amdgcn_readfirstlane((int)cls_s[wave][r][kb]);
-            const bool uni = uniform_row[r];
-            if (cls & 0x80) {                    // no valid key in this block
-                if (!(uni && (cls & 1))) continue;
-                cls = 1;                         // uniform row: masked real keys take part
-            }
-            const bf16x8 k0 = kf[frag_index(a, h, kb, 0, nb, lane)];
-            const bf16x8 k1 = kf[frag_index(a, h, kb, 1, nb, lane)];
-            const bf16x8 v0 = vf[frag_index(a, h, kb, 0, nb, lane)];
-            const bf16x8 v1 = vf[frag_index(a, h, kb, 1, nb, lane)];
-            f32x16 s = mfma32(k0, q0[r], bias);
-            s = mfma32(k1, q1[r], s);
-            if (cls != 2) {
-                // this lane's keys: 8*(v/4) + 4*half + (v%4) -> one dword of codes per group of 4
-                const uint32_t* cw = reinterpret_cast<const uint32_t*>(
-                    codes + (size_t)a * nb * 32 + kb * 32 + 4 * half);
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const uint32_t w = cw[2 * g];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t code = (w >> (8 * e)) & 0xffu;
-                        const int v = 4 * g + e;
-                        if (uni) s[v] = code == 1 ? 0.f : -INFINITY;
-                        else if (code != 2) s[v] = -INFINITY;
-                    }
-                }
-            }
-            float mx = s[0];
-#pragma unroll
-            for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
-            mx = xhalf_max(mx);
-            const float m_new = fmaxf(m[r], mx);
-            const float alpha = fast_exp2(m[r] - m_new);
-            m[r] = m_new;
-            float ls = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) { s[v] = fast_exp2(s[v] - m_new); ls += s[v]; }
-            l[r] = l[r] * alpha + ls;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o[r][v] *= alpha;
-            bf16x8 p0, p1;
-            acc_to_frags(s, p0, p1);
-            o[r] = mfma32(v0, p0, o[r]);
-            o[r] = mfma32(v1, p1, o[r]);
-        }
-    }
-
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        if (a0 + r < N) {
-            const int a = a0 + r;
-            const float inv = fast_rcp(xhalf_sum(l[r]));
-            const u32x4 g0 = __builtin_bit_cast(u32x4, gf[frag_index(a, h, qb, 0, nb, lane)]);
-            const u32x4 g1 = __builtin_bit_cast(u32x4, gf[frag_index(a, h, qb, 1, nb, lane)]);
-            f32x16 og;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                og[2 * e] = o[r][2 * e] * inv * bf16_lo(g0[e]);
-                og[2 * e + 1] = o[r][2 * e + 1] * inv * bf16_hi(g0[e]);
-                og[8 + 2 * e] = o[r][8 + 2 * e] * inv * bf16_lo(g1[e]);
-                og[8 + 2 * e + 1] = o[r][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
-            }
-            bf16x8 f0, f1;
-            acc_to_frags(og, f0, f1);
-            of[frag_index(a, h, qb, 0, nb, lane)] = f0;
-            of[frag_index(a, h, qb, 1, nb, lane)] = f1;
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
 // output projection: out'[a][b] = W_o (gated o), 64 positions per wavefront
 // ------------------------------------------------------------------------------------------
 template <int IO>
@@ -422,13 +270,11 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
         hipLaunchKernelGGL(triattn_proj_kernel<KFH_BF16>, grid_rows, block, 0, stream, x, mask, blob,
                            qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
 
-    constexpr int R = 4;
-    const int qgroups = (nb + 3) / 4;
-    const int nchunks = kH * ((N + R - 1) / R);
-    const int nslots = ((nchunks + 7) / 8) * qgroups;
-    hipLaunchKernelGGL(triattn_flash_kernel<R>, dim3(nslots * 8), block, 0, stream, qf, kf, vf, gf,
-                       reinterpret_cast<const f32x4*>(ws.biasf), ws.codes, of, N, nb, qgroups,
-                       nchunks);
+    FlashArgs fa{};
+    fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = gf; fa.of = of;
+    fa.biasf = ws.biasf; fa.codes = ws.codes;
+    fa.nrows = N; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
+    launch_flash(fa, 32, stream);
 
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, block, 0, stream, of, blob,

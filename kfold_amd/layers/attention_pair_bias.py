@@ -1,0 +1,136 @@
+"""Self attention with pair bias, ``hip`` backend.
+
+``SelfAttentionPairBias`` mirrors the reference module
+(src/kfold/model/layers/folding/attention_pair_bias.py:70-158; parameters of
+``AttentionPairBias`` :30-67 and ``AdaLN`` model/primitives/normalization.py:94-115).
+``hip_attention_pair_bias`` is what a ``kernel_backend == "hip"`` branch of
+``attention_pair_bias`` (model/primitives/attention.py:62-66) would call, next to
+``triton_attention_pair_bias``: it receives already normalised ``x_q``/``x_k``.
+
+Only self attention (``x_q is x_k``, Lq == Lk) is built; the local-window
+``CrossAttentionPairBias`` of the diffusion atom transformer is out of scope.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .. import ops
+from ..primitives._common import cache_key, cached_blob, check_inference
+from ..primitives.layers import LayerNorm, Linear, LinearNoBias
+
+
+def _parameters(module: nn.Module):
+    cond = getattr(module, "use_single_conditioning", False)
+    p = dict(q_w=module.linear_q.weight, q_b=module.linear_q.bias, k_w=module.linear_k.weight,
+             v_w=module.linear_v.weight, g_w=module.linear_g.weight, o_w=module.linear_out.weight)
+    if cond:
+        ada = module.adaln_a
+        p.update(adaln_s_w=ada.layernorm_s.weight, adaln_g_w=ada.linear_g.weight,
+                 adaln_g_b=ada.linear_g.bias, adaln_bias_w=ada.linear_bias.weight,
+                 ada_out_w=module.linear_ada_out.weight, ada_out_b=module.linear_ada_out.bias)
+    elif hasattr(module, "layernorm_a"):
+        p.update(ln_w=module.layernorm_a.weight, ln_b=module.layernorm_a.bias)
+    return p
+
+
+def _cond_channels(module: nn.Module) -> int:
+    if getattr(module, "use_single_conditioning", False):
+        return module.linear_ada_out.weight.shape[1]
+    return 0
+
+
+def _flatten(t: torch.Tensor, keep: int, lead: torch.Size):
+    """Flatten the leading dims of ``t`` (which broadcast against ``lead``) to 1 or prod(lead)."""
+    tl = t.shape[:t.dim() - keep]
+    if all(d == 1 for d in tl):
+        return t.reshape((1,) + t.shape[t.dim() - keep:]), False
+    full = torch.broadcast_to(t, tuple(lead) + t.shape[t.dim() - keep:])
+    return full.reshape((-1,) + t.shape[t.dim() - keep:]), True
+
+
+def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
+    check_inference(a, "pair-bias attention")
+    if module.linear_g.bias is not None or module.linear_out.bias is not None:
+        raise NotImplementedError("hip pair-bias attention: gate / output projection biases")
+    params = _parameters(module)
+    C, H, Cs = module.channel_a, module.num_heads, _cond_channels(module)
+    key = cache_key(tuple(params.values()), a, torch.bfloat16)
+    blob = cached_blob(module, "_hip_apb_cache", key,
+                       lambda: ops.apb_pack(C, H, Cs, device=a.device, **params))
+    lead = a.shape[:-2]
+    io = a if a.dtype in (torch.bfloat16, torch.float32) else a.float()
+    af = io.reshape((-1,) + a.shape[-2:])
+    pb, per_sample = _flatten(pair_bias, 3, lead)
+    mk, _ = _flatten(mask, 1, lead)
+    sf = None
+    if s is not None and apply_norm and Cs:
+        sf, _ = _flatten(s, 2, lead)
+    tiles = ops.bias_tiles_from_dense(pb)
+    out = ops.apb_forward(af, sf, tiles, mk, blob, H, Cs, apply_norm, per_sample and af.shape[0] > 1,
+                          eps=1e-5)
+    return out.reshape(a.shape).to(a.dtype)
+
+
+@torch.compiler.disable
+def hip_attention_pair_bias(module: nn.Module, x_q: torch.Tensor, x_k: torch.Tensor,
+                            pair_bias: torch.Tensor, mask: torch.Tensor, *,
+                            call_site: str = "confidence") -> torch.Tensor:
+    """x_q, x_k [*, L, C] normalised (must be the same tensor), pair_bias broadcastable to
+    [*, H, L, L], mask broadcastable to [*, L]."""
+    if x_q is not x_k and (x_q.shape != x_k.shape or x_q.data_ptr() != x_k.data_ptr()):
+        raise NotImplementedError("hip pair-bias attention is built for self attention only")
+    return _run(module, x_q, None, pair_bias, mask, apply_norm=False)
+
+
+class AdaLN(nn.Module):
+    """Parameter holder, names of model/primitives/normalization.py:94-115."""
+
+    def __init__(self, channel_a: int, channel_s: int):
+        super().__init__()
+        self.layernorm_a = LayerNorm(channel_a, create_scale=False, create_offset=False)
+        self.layernorm_s = LayerNorm(channel_s, create_scale=True, create_offset=False)
+        self.linear_g = Linear(channel_s, channel_a, init="gating")
+        self.linear_bias = LinearNoBias(channel_s, channel_a, init="final")
+
+
+class SelfAttentionPairBias(nn.Module):
+    def __init__(self, channel_a: int, num_heads: int, channel_s: int | None, call_site: str,
+                 inf: float = 1e9, kernel_backend: str = "hip") -> None:
+        super().__init__()
+        if kernel_backend != "hip":
+            raise ValueError(
+                f"kfold_amd implements kernel_backend='hip' only, got {kernel_backend!r}")
+        if call_site not in {"diffusion_global", "confidence"}:
+            raise ValueError(f"Unsupported self APB call site: {call_site!r}")
+        assert channel_a % num_heads == 0
+        self.use_single_conditioning = channel_s is not None
+        self.call_site = call_site
+        self.channel_a = channel_a
+        self.num_heads = num_heads
+        self.head_dim = channel_a // num_heads
+        self.inf = inf
+        self.kernel_backend = kernel_backend
+        self.linear_q = Linear(channel_a, channel_a, init="default")
+        self.linear_k = LinearNoBias(channel_a, channel_a, init="default")
+        self.linear_v = LinearNoBias(channel_a, channel_a, init="default")
+        self.linear_g = LinearNoBias(channel_a, channel_a, init="gating")
+        self.linear_out = LinearNoBias(channel_a, channel_a,
+                                       init="default" if self.use_single_conditioning else "final")
+        if self.use_single_conditioning:
+            self.adaln_a = AdaLN(channel_a, channel_s)
+            self.linear_ada_out = Linear(channel_s, channel_a, init="gating")
+            with torch.no_grad():
+                self.linear_ada_out.bias.fill_(-2.0)      # the reference's "gating_closed"
+        else:
+            self.layernorm_a = LayerNorm(channel_a, create_offset=True)
+
+    def forward(self, a: torch.Tensor, s: torch.Tensor | None, pair_bias: torch.Tensor,
+                mask: torch.Tensor) -> torch.Tensor:
+        """a [..., L, c_a], s [..., L, c_s] or None, pair_bias [..., H, L, L], mask [..., L]."""
+        if self.use_single_conditioning:
+            assert s is not None
+        else:
+            assert s is None
+        return _run(self, a, s, pair_bias, mask, apply_norm=True)

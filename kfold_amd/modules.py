@@ -1,0 +1,161 @@
+"""Pairformer block / trunk composition on the hip backend.
+
+``PairformerBlock`` mirrors the reference's pair track
+(src/kfold/model/modules/apo_module.py:107-172); ``PairSingleBlock`` adds the single track
+of ``ConfidencePairSingleBlock.forward`` (model/modules/confidence_head.py:161-175) on top,
+which is the block the benchmark configs are quoted on; ``TriangularBlock`` mirrors the
+shipping trunk block (model/modules/tri_stack.py:96-151, no triangle attention).
+
+Residual adds are fused into the producing kernels (``z += update`` happens in the output
+phase of each op, in place on the caller's tensor like the reference's eval-mode
+``z.add_``), and the block's final ``z * pair_mask`` is fused into the transition kernel.
+"""
+
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from . import ops
+from .layers.attention_pair_bias import SelfAttentionPairBias, _cond_channels, _parameters
+from .layers.transition import Transition, hip_transition
+from .primitives._common import cache_key, cached_blob, check_inference
+from .primitives.layers import LayerNorm, LinearNoBias
+from .primitives.triangle_attention import (
+    TriangleAttentionEndingNode,
+    TriangleAttentionStartingNode,
+)
+from .primitives.triangle_attention import _parameters as _ta_parameters
+from .primitives.triangle_multiplication import (
+    TriangleMultiplicationIncoming,
+    TriangleMultiplicationOutgoing,
+)
+from .primitives.triangle_multiplication import _parameters as _tm_parameters
+
+
+def _contiguous_io(t: torch.Tensor, name: str) -> None:
+    if not t.is_contiguous():
+        raise ValueError(f"{name} must be contiguous for the in-place hip block")
+    if t.dtype not in (torch.bfloat16, torch.float32):
+        raise TypeError(f"{name}: the hip block runs on bfloat16 or float32 tensors, got {t.dtype}")
+
+
+def _trimul_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None:
+    params = _tm_parameters(mod)
+    blob = cached_blob(mod, "_hip_multiplication_cache", cache_key(params, z, torch.bfloat16),
+                       lambda: ops.trimul_pack(*params, device=z.device))
+    ops.trimul_forward(z, mask, blob, mod.direction, eps=mod.layernorm_in.eps, residual=z, out=z)
+
+
+def _triattn_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None:
+    params = _ta_parameters(mod)
+    blob = cached_blob(mod, "_hip_attention_cache", cache_key(params, z, torch.bfloat16),
+                       lambda: ops.triattn_pack(*params, device=z.device))
+    ops.triattn_forward(z, mask, blob, mod.no_heads, mod.starting, eps=mod.layer_norm.eps,
+                        residual=z, out=z)
+
+
+class PairformerBlock(nn.Module):
+    """tri-mul out, tri-mul in, tri-attn start, tri-attn end, transition(x2), final mask."""
+
+    def __init__(self, channel_z: int = 128, num_tri_heads: int = 4, dropout: float = 0.1,
+                 kernel_backend: str = "hip"):
+        super().__init__()
+        self.kernel_backend = kernel_backend
+        self.channel_z = channel_z
+        self.tri_mul_out = TriangleMultiplicationOutgoing(channel_z, kernel_backend=kernel_backend)
+        self.tri_mul_in = TriangleMultiplicationIncoming(channel_z, kernel_backend=kernel_backend)
+        self.tri_att_start = TriangleAttentionStartingNode(channel_z, num_tri_heads,
+                                                           kernel_backend=kernel_backend)
+        self.tri_att_end = TriangleAttentionEndingNode(channel_z, num_tri_heads,
+                                                       kernel_backend=kernel_backend)
+        self.transition_z = Transition(channel_z, expansion_factor=2)
+
+    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor, inplace_output: bool = False) -> torch.Tensor:
+        """z [B, N, N, C] is updated in place by the four triangle ops (as the reference does in
+        eval mode); returns ``(z + transition(z)) * pair_mask`` as a new tensor, or written over
+        ``z`` when ``inplace_output`` is set."""
+        check_inference(z, "Pairformer block")
+        if self.training:
+            raise RuntimeError("The hip Pairformer block is inference-only (call .eval()).")
+        _contiguous_io(z, "z")
+        _trimul_inplace(self.tri_mul_out, z, pair_mask)
+        _trimul_inplace(self.tri_mul_in, z, pair_mask)
+        _triattn_inplace(self.tri_att_start, z, pair_mask)
+        _triattn_inplace(self.tri_att_end, z, pair_mask)
+        return hip_transition(self.transition_z, z, residual=z, mask=pair_mask,
+                              out=z if inplace_output else None)
+
+
+class TriangularBlock(nn.Module):
+    """tri-mul out, tri-mul in, transition(x4); no triangle attention, no final mask."""
+
+    def __init__(self, channel_z: int = 128, dropout: float = 0.25, kernel_backend: str = "hip"):
+        super().__init__()
+        self.kernel_backend = kernel_backend
+        self.channel_z = channel_z
+        self.tri_mul_out = TriangleMultiplicationOutgoing(channel_z, kernel_backend=kernel_backend)
+        self.tri_mul_in = TriangleMultiplicationIncoming(channel_z, kernel_backend=kernel_backend)
+        self.transition_z = Transition(channel_z, expansion_factor=4)
+
+    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor) -> torch.Tensor:
+        check_inference(z, "triangular block")
+        if self.training:
+            raise RuntimeError("The hip triangular block is inference-only (call .eval()).")
+        _contiguous_io(z, "z")
+        _trimul_inplace(self.tri_mul_out, z, pair_mask)
+        _trimul_inplace(self.tri_mul_in, z, pair_mask)
+        return hip_transition(self.transition_z, z, residual=z, out=z)
+
+
+class PairSingleBlock(nn.Module):
+    """Pair track (``PairformerBlock``) followed by the single track: pair bias from z,
+    ``s += SelfAttentionPairBias(s)``, ``s += Transition_4(s)``."""
+
+    def __init__(self, channel_s: int = 384, channel_z: int = 128, num_heads: int = 16,
+                 num_tri_heads: int = 4, kernel_backend: str = "hip"):
+        super().__init__()
+        self.kernel_backend = kernel_backend
+        self.num_heads = num_heads
+        self.pair_block = PairformerBlock(channel_z, num_tri_heads, kernel_backend=kernel_backend)
+        self.layernorm_z = LayerNorm(channel_z)
+        self.linear_pair_bias = LinearNoBias(channel_z, num_heads)
+        self.attention = SelfAttentionPairBias(channel_s, num_heads, None, call_site="confidence",
+                                               kernel_backend=kernel_backend)
+        self.transition = Transition(channel_s, expansion_factor=4)
+
+    def forward(self, z: torch.Tensor, s: torch.Tensor, pair_mask: torch.Tensor, mask: torch.Tensor,
+                inplace_output: bool = False):
+        """z [B, N, N, Cz], s [B, N, Cs], pair_mask [B, N, N], mask [B, N]; s is updated in place."""
+        _contiguous_io(s, "s")
+        z = self.pair_block(z, pair_mask, inplace_output=inplace_output)
+        B = z.shape[0]
+        pb_params = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_pair_bias.weight)
+        pb_blob = cached_blob(self, "_hip_pair_bias_cache", cache_key(pb_params, z, torch.bfloat16),
+                              lambda: ops.pair_bias_pack(*pb_params, device=z.device))
+        tiles = ops.pair_bias_project(z, pb_blob, self.num_heads, eps=self.layernorm_z.eps)
+        att = self.attention
+        params = _parameters(att)
+        blob = cached_blob(att, "_hip_apb_cache", cache_key(tuple(params.values()), s, torch.bfloat16),
+                           lambda: ops.apb_pack(att.channel_a, att.num_heads, _cond_channels(att),
+                                                device=s.device, **params))
+        ops.apb_forward(s, None, tiles, mask.reshape(B, -1), blob, att.num_heads, 0, True, B > 1,
+                        eps=att.layernorm_a.eps, residual=s, out=s)
+        hip_transition(self.transition, s, residual=s, out=s)
+        return z, s
+
+
+class PairformerTrunk(nn.Module):
+    """A stack of ``PairSingleBlock``; z and s are updated in place block after block."""
+
+    def __init__(self, num_blocks: int, channel_s: int = 384, channel_z: int = 128,
+                 num_heads: int = 16, num_tri_heads: int = 4, kernel_backend: str = "hip"):
+        super().__init__()
+        self.blocks = nn.ModuleList(
+            PairSingleBlock(channel_s, channel_z, num_heads, num_tri_heads, kernel_backend)
+            for _ in range(num_blocks))
+
+    def forward(self, z, s, pair_mask, mask):
+        for blk in self.blocks:
+            z, s = blk(z, s, pair_mask, mask, inplace_output=True)
+        return z, s

@@ -162,3 +162,153 @@ def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tens
                                     out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C, heads,
                                     0 if starting else 1, float(eps), _io_dtype(xc), _stream(dev)))
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# transition
+# ---------------------------------------------------------------------------------------
+def transition_pack(ln_w, ln_b, swiglu_w, out_w, device: torch.device) -> torch.Tensor:
+    L = _lib.lib()
+    C = out_w.shape[0]
+    E = out_w.shape[1] // C
+    nbytes = L.kfh_transition_packed_bytes(C, E)
+    if nbytes == 0:
+        raise NotImplementedError(f"hip transition does not support C={C}, expansion={E}")
+    ws = _weights_f32(device, ln_w, ln_b, swiglu_w, out_w)
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        check(L.kfh_transition_pack(*[_ptr(w) for w in ws], KFH_F32, C, E, blob.data_ptr(),
+                                    _stream(device)))
+    return blob
+
+
+def transition_forward(x: torch.Tensor, blob: torch.Tensor, expansion: int, eps: float = 1e-5,
+                       residual: torch.Tensor | None = None, mask: torch.Tensor | None = None,
+                       out: torch.Tensor | None = None) -> torch.Tensor:
+    """``out = ((residual or 0) + Transition(x)) * (mask or 1)`` over the last dim of x."""
+    dev = _require_cuda(x, blob, residual, mask, out)
+    C = x.shape[-1]
+    rows = x.numel() // C if x.numel() else 0
+    xc = x.contiguous()
+    if out is None:
+        out = torch.empty_like(xc)
+    elif out.shape != x.shape or out.dtype != x.dtype or not out.is_contiguous():
+        raise ValueError("out must be contiguous with the shape and dtype of x")
+    if residual is not None and (residual.shape != x.shape or residual.dtype != x.dtype
+                                 or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous with the shape and dtype of x")
+    m8 = None if mask is None else _mask_bytes(mask, x.shape[:-1])
+    if rows == 0:
+        return out
+    L = _lib.lib()
+    ws_bytes = L.kfh_transition_workspace_bytes(rows, C, expansion)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    with torch.cuda.device(dev):
+        check(L.kfh_transition_forward(xc.data_ptr(), blob.data_ptr(), _ptr(residual), _ptr(m8),
+                                       out.data_ptr(), _ptr(ws), ws_bytes, rows, C, expansion,
+                                       float(eps), _io_dtype(xc), _stream(dev)))
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# pair bias tiles and pair-bias attention
+# ---------------------------------------------------------------------------------------
+def bias_tiles_from_dense(pair_bias: torch.Tensor) -> torch.Tensor:
+    """Dense pair bias [nbatch, H, L, L] -> the attention kernel's fp32 tiles (flat uint8)."""
+    dev = _require_cuda(pair_bias)
+    nbatch, H, Lq, Lk = pair_bias.shape
+    if Lq != Lk:
+        raise NotImplementedError("hip pair-bias attention is built for self attention (Lq == Lk)")
+    pb = pair_bias.contiguous()
+    if pb.dtype not in _IO_DTYPES:
+        pb = pb.float()
+    L = _lib.lib()
+    tiles = torch.empty(L.kfh_bias_tiles_bytes(nbatch, H, Lq), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(L.kfh_bias_tiles_from_dense(pb.data_ptr(), _io_dtype(pb), tiles.data_ptr(), nbatch, H, Lq,
+                                          _stream(dev)))
+    return tiles
+
+
+def pair_bias_pack(ln_w, ln_b, w, device: torch.device) -> torch.Tensor:
+    L = _lib.lib()
+    H, C = w.shape
+    nbytes = L.kfh_pair_bias_packed_bytes(C, H)
+    if nbytes == 0:
+        raise NotImplementedError(f"hip pair-bias projection is built for C=128, H<=32; got C={C}, H={H}")
+    ws = _weights_f32(device, ln_w, ln_b, w)
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        check(L.kfh_pair_bias_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, blob.data_ptr(), _stream(device)))
+    return blob
+
+
+def pair_bias_project(z: torch.Tensor, blob: torch.Tensor, heads: int, eps: float = 1e-5) -> torch.Tensor:
+    """tiles of ``linear_pair_bias(LN(z))`` for z [B, N, N, C]; returns the flat tile buffer."""
+    dev = _require_cuda(z, blob)
+    B, N, N2, C = z.shape
+    assert N == N2
+    zc = z.contiguous()
+    L = _lib.lib()
+    tiles = torch.empty(L.kfh_bias_tiles_bytes(B, heads, N), dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(L.kfh_pair_bias_project(zc.data_ptr(), blob.data_ptr(), tiles.data_ptr(), B, N, C, heads,
+                                      float(eps), _io_dtype(zc), _stream(dev)))
+    return tiles
+
+
+def apb_pack(C: int, H: int, Cs: int, *, ln_w=None, ln_b=None, q_w, q_b, k_w, v_w, g_w, o_w,
+             adaln_s_w=None, adaln_g_w=None, adaln_g_b=None, adaln_bias_w=None, ada_out_w=None,
+             ada_out_b=None, device: torch.device) -> torch.Tensor:
+    L = _lib.lib()
+    nbytes = L.kfh_apb_packed_bytes(C, H, Cs)
+    if nbytes == 0:
+        raise NotImplementedError(
+            f"hip pair-bias attention: C={C}, H={H}, Cs={Cs} unsupported "
+            "(channels multiples of 128 up to 2048, head dim <= 64)")
+    ws = _weights_f32(device, ln_w, ln_b, q_w, q_b, k_w, v_w, g_w, o_w, adaln_s_w, adaln_g_w,
+                      adaln_g_b, adaln_bias_w, ada_out_w, ada_out_b)
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        check(L.kfh_apb_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, Cs, blob.data_ptr(), _stream(device)))
+    return blob
+
+
+def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tensor, mask: torch.Tensor,
+                blob: torch.Tensor, heads: int, cond_channels: int, apply_norm: bool,
+                bias_per_sample: bool, eps: float = 1e-5, residual: torch.Tensor | None = None,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """a [S, L, C]; s_cond [S or 1, L, Cs] or None; mask [S or 1, L]; tiles from the calls above."""
+    dev = _require_cuda(a, s_cond, tiles, mask, blob, residual, out)
+    S, Lq, C = a.shape
+    ac = a.contiguous()
+    m8 = _mask_bytes(mask, mask.shape)
+    if m8.shape not in ((S, Lq), (1, Lq)):
+        raise ValueError(f"mask shape {tuple(mask.shape)} does not match a {tuple(a.shape)}")
+    sc = None
+    if s_cond is not None:
+        sc = s_cond.contiguous()
+        if sc.dtype != ac.dtype:
+            sc = sc.to(ac.dtype)
+        if sc.shape[0] not in (1, S) or sc.shape[1] != Lq or sc.shape[2] != cond_channels:
+            raise ValueError(f"s shape {tuple(s_cond.shape)} does not match a {tuple(a.shape)}")
+    if out is None:
+        out = torch.empty_like(ac)
+    elif out.shape != a.shape or out.dtype != a.dtype or not out.is_contiguous():
+        raise ValueError("out must be contiguous with the shape and dtype of a")
+    if residual is not None and (residual.shape != a.shape or residual.dtype != a.dtype
+                                 or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous with the shape and dtype of a")
+    L = _lib.lib()
+    ws_bytes = L.kfh_apb_workspace_bytes(S, Lq, C, heads, cond_channels)
+    if ws_bytes == 0:
+        raise NotImplementedError(f"hip pair-bias attention: unsupported shape S={S} L={Lq} C={C} H={heads}")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(L.kfh_apb_forward(ac.data_ptr(), _ptr(sc), tiles.data_ptr(), m8.data_ptr(), blob.data_ptr(),
+                                _ptr(residual), out.data_ptr(), ws.data_ptr(), ws_bytes, S, Lq, C, heads,
+                                cond_channels, 1 if apply_norm else 0, 1 if bias_per_sample else 0,
+                                1 if m8.shape[0] == S and S > 1 else 0,
+                                1 if sc is not None and sc.shape[0] == S and S > 1 else 0,
+                                float(eps), _io_dtype(ac), _stream(dev)))
+    return out

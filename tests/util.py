@@ -23,8 +23,15 @@ def errors(out: torch.Tensor, ref: torch.Tensor) -> dict:
     }
 
 
-def assert_close(out, ref, what="", max_abs=MAX_ABS, mean_abs=MEAN_ABS, rel_fro=REL_FRO):
+def assert_close(out, ref, what="", max_abs=MAX_ABS, mean_abs=MEAN_ABS, rel_fro=REL_FRO,
+                 auto_scale=False):
+    """``auto_scale``: for stress cases whose weights are larger than the benchmark's std 0.02
+    the outputs are O(1) instead of O(0.1); the absolute tolerances (stated for the benchmark
+    scale) then grow with the reference RMS, the relative gate stays as is."""
     e = errors(out, ref)
+    if auto_scale:
+        f = max(1.0, ref.detach().float().pow(2).mean().sqrt().item() / 0.2)
+        max_abs, mean_abs = max_abs * f, mean_abs * f
     msg = f"{what}: {e}"
     assert e["finite"], msg
     assert e["max_abs"] <= max_abs, msg
