@@ -44,6 +44,12 @@ extern "C" {
 #define KFH_OUTGOING 0
 #define KFH_INCOMING 1
 
+/* stage selectors of the *_forward_stages() entry points */
+#define KFH_STAGE_IN 1   /* LayerNorm + input projections                      */
+#define KFH_STAGE_CORE 2 /* the contraction (tri-mul) / the attention (tri-attn) */
+#define KFH_STAGE_OUT 4  /* output projection, gate, residual                   */
+#define KFH_STAGE_ALL 7
+
 int kfh_version(void);
 const char* kfh_last_error(void);
 
@@ -75,6 +81,14 @@ int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, con
                        void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                        int direction, float eps, int io_dtype, void* stream);
 
+/* Same as kfh_trimul_forward but runs only the kernels selected by `stages` (an OR of
+ * KFH_STAGE_*); later stages read what earlier ones left in `workspace`.  For profiling and
+ * benchmarks of the individual kernels; no counterpart in the reference. */
+int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* blob,
+                              const void* residual, void* out, void* workspace,
+                              size_t workspace_bytes, int B, int N, int C, int direction, float eps,
+                              int io_dtype, int stages, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Triangle attention around the starting / ending node (Algorithms 14/15).
  * Replaces kernels/triton/triangle_attention/ops.py:24 `precompute` and :56 `forward` as
@@ -101,6 +115,12 @@ size_t kfh_triattn_workspace_bytes(int N, int C, int H);
 int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, const void* residual,
                         void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                         int H, int ending, float eps, int io_dtype, void* stream);
+
+/* Stage-selective variant, see kfh_trimul_forward_stages. */
+int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* blob,
+                               const void* residual, void* out, void* workspace,
+                               size_t workspace_bytes, int B, int N, int C, int H, int ending,
+                               float eps, int io_dtype, int stages, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Transition (Algorithm 11, SwiGLU).  Replaces the torch modules

@@ -14,6 +14,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libkfold_hip.so"
 
 KFH_BF16, KFH_F32 = 0, 1
 KFH_OUTGOING, KFH_INCOMING = 0, 1
+KFH_STAGE_IN, KFH_STAGE_CORE, KFH_STAGE_OUT, KFH_STAGE_ALL = 1, 2, 4, 7
 
 # name -> (restype, argtypes); mirrors include/kfold_hip.h one to one
 _P = c_void_p
@@ -25,6 +26,10 @@ SIGNATURES: dict[str, tuple] = {
     "kfh_trimul_workspace_bytes": (c_size_t, [c_int, c_int]),
     "kfh_trimul_forward": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                    c_float, c_int, _P]),
+    "kfh_trimul_forward_stages": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
+                                          c_float, c_int, c_int, _P]),
+    "kfh_triattn_forward_stages": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
+                                           c_int, c_float, c_int, c_int, _P]),
     "kfh_triattn_packed_bytes": (c_size_t, [c_int, c_int]),
     "kfh_triattn_pack": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P]),
     "kfh_triattn_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),

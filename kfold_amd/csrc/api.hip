@@ -62,7 +62,15 @@ size_t kfh_trimul_workspace_bytes(int N, int C) {
 
 int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, const void* residual,
                        void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
-                       int direction, float eps, int io_dtype, void* stream_) {
+                       int direction, float eps, int io_dtype, void* stream) {
+    return kfh_trimul_forward_stages(z, mask, blob, residual, out, workspace, workspace_bytes, B, N, C,
+                                     direction, eps, io_dtype, KFH_STAGE_ALL, stream);
+}
+
+int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* blob,
+                              const void* residual, void* out, void* workspace,
+                              size_t workspace_bytes, int B, int N, int C, int direction, float eps,
+                              int io_dtype, int stages, void* stream_) {
     if (C != kC) return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d, only C=128 is built", C);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "trimul_forward: bad shape B=%d N=%d", B, N);
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "trimul_forward: bad io_dtype %d", io_dtype);
@@ -89,10 +97,13 @@ int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, con
         const char* zb = static_cast<const char*>(z) + off;
         const char* rb = residual ? static_cast<const char*>(residual) + off : nullptr;
         char* ob = static_cast<char*>(out) + off;
-        launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, gate, N, np,
-                         direction == KFH_INCOMING, eps, stream);
-        launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream);
-        launch_trimul_out(planes_y, gate, bl, rb, ob, io_dtype, N, np, eps, stream);
+        if (stages & KFH_STAGE_IN)
+            launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, gate, N, np,
+                             direction == KFH_INCOMING, eps, stream);
+        if (stages & KFH_STAGE_CORE)
+            launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream);
+        if (stages & KFH_STAGE_OUT)
+            launch_trimul_out(planes_y, gate, bl, rb, ob, io_dtype, N, np, eps, stream);
     }
     return check_launch("trimul_forward");
 }
@@ -155,7 +166,15 @@ size_t kfh_triattn_workspace_bytes(int N, int C, int H) {
 
 int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, const void* residual,
                         void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
-                        int H, int ending, float eps, int io_dtype, void* stream_) {
+                        int H, int ending, float eps, int io_dtype, void* stream) {
+    return kfh_triattn_forward_stages(x, mask, blob, residual, out, workspace, workspace_bytes, B, N, C,
+                                      H, ending, eps, io_dtype, KFH_STAGE_ALL, stream);
+}
+
+int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* blob,
+                               const void* residual, void* out, void* workspace,
+                               size_t workspace_bytes, int B, int N, int C, int H, int ending,
+                               float eps, int io_dtype, int stages, void* stream_) {
     if (C != kC || H != 4)
         return fail(KFH_EUNSUPPORTED, "triattn_forward: C=%d H=%d, only C=128 H=4 is built", C, H);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "triattn_forward: bad shape B=%d N=%d", B, N);
@@ -178,7 +197,7 @@ int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, co
     const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
     for (int b = 0; b < B; ++b) {
         const size_t off = (size_t)b * N * N * C * esz;
-        if (N % 32) {
+        if ((stages & KFH_STAGE_IN) && N % 32) {
             // queries beyond N in the last query block have no projected bias: keep their tiles finite
             for (int h = 0; h < 4; ++h)
                 launch_fill_zero(ws.biasf + (((size_t)h * sz.nb + (sz.nb - 1)) * sz.nb) * 1024,
@@ -187,7 +206,7 @@ int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, co
         launch_triattn(static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N,
                        static_cast<const char*>(blob), ws,
                        residual ? static_cast<const char*>(residual) + off : nullptr,
-                       static_cast<char*>(out) + off, N, ending, eps, stream);
+                       static_cast<char*>(out) + off, N, ending, eps, stages, stream);
     }
     return check_launch("triattn_forward");
 }

@@ -74,7 +74,7 @@ int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
 void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream);
 void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
-                    float eps, hipStream_t stream);
+                    float eps, int stages, hipStream_t stream);
 
 // ---- pair transition (transition.hip) ----------------------------------------------------
 // Packed blob (C = 128, expansion E): 4E steps x 24 KiB { u block, v block, W_out slice of the

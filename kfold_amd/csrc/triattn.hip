@@ -255,7 +255,7 @@ __global__ __launch_bounds__(256) void triattn_out_kernel(
 // ------------------------------------------------------------------------------------------
 void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
-                    float eps, hipStream_t stream) {
+                    float eps, int stages, hipStream_t stream) {
     const int nb = (N + 31) / 32;
     bf16x8* qf = static_cast<bf16x8*>(ws.qf);
     bf16x8* kf = static_cast<bf16x8*>(ws.kf);
@@ -263,18 +263,21 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
     bf16x8* gf = static_cast<bf16x8*>(ws.gf);
     bf16x8* of = static_cast<bf16x8*>(ws.of);
     dim3 grid_rows((N + kTileA - 1) / kTileA, N), block(256);
-    if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(triattn_proj_kernel<KFH_F32>, grid_rows, block, 0, stream, x, mask, blob, qf,
-                           kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
-    else
-        hipLaunchKernelGGL(triattn_proj_kernel<KFH_BF16>, grid_rows, block, 0, stream, x, mask, blob,
-                           qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+    if (stages & KFH_STAGE_IN) {
+        if (io_dtype == KFH_F32)
+            hipLaunchKernelGGL(triattn_proj_kernel<KFH_F32>, grid_rows, block, 0, stream, x, mask, blob,
+                               qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+        else
+            hipLaunchKernelGGL(triattn_proj_kernel<KFH_BF16>, grid_rows, block, 0, stream, x, mask, blob,
+                               qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+    }
 
     FlashArgs fa{};
     fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = gf; fa.of = of;
     fa.biasf = ws.biasf; fa.codes = ws.codes;
     fa.nrows = N; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
-    launch_flash(fa, 32, stream);
+    if (stages & KFH_STAGE_CORE) launch_flash(fa, 32, stream);
+    if (!(stages & KFH_STAGE_OUT)) return;
 
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, block, 0, stream, of, blob,
