@@ -117,7 +117,7 @@ TaSizes ta_sizes(int N) {
     TaSizes s;
     s.nb = (N + 31) / 32;
     s.frag = align_up((size_t)N * 4 * s.nb * 2048);
-    s.bias = align_up((size_t)4 * s.nb * s.nb * 4096);
+    s.bias = align_up((size_t)4 * s.nb * s.nb * 2048);
     s.codes = align_up((size_t)N * s.nb * 32);
     s.total = 5 * s.frag + s.bias + s.codes;
     return s;
@@ -192,7 +192,7 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
     TriattnWorkspace ws;
     ws.qf = w; ws.kf = w + sz.frag; ws.vf = w + 2 * sz.frag; ws.gf = w + 3 * sz.frag;
     ws.of = w + 4 * sz.frag;
-    ws.biasf = reinterpret_cast<float*>(w + 5 * sz.frag);
+    ws.biast = reinterpret_cast<uint16_t*>(w + 5 * sz.frag);
     ws.codes = reinterpret_cast<uint8_t*>(w + 5 * sz.frag + sz.bias);
     const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
     for (int b = 0; b < B; ++b) {
@@ -200,8 +200,8 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
         if ((stages & KFH_STAGE_IN) && N % 32) {
             // queries beyond N in the last query block have no projected bias: keep their tiles finite
             for (int h = 0; h < 4; ++h)
-                launch_fill_zero(ws.biasf + (((size_t)h * sz.nb + (sz.nb - 1)) * sz.nb) * 1024,
-                                 (size_t)sz.nb * 4096, stream);
+                launch_fill_zero(ws.biast + (((size_t)h * sz.nb + (sz.nb - 1)) * sz.nb) * kBiasTileElems,
+                                 (size_t)sz.nb * 2048, stream);
         }
         launch_triattn(static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N,
                        static_cast<const char*>(blob), ws,

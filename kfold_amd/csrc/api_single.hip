@@ -92,7 +92,7 @@ extern "C" {
 size_t kfh_bias_tiles_bytes(int nbatch, int H, int L) {
     if (nbatch <= 0 || H <= 0 || L <= 0) return 0;
     const size_t nb = (L + 31) / 32;
-    return align_up((size_t)nbatch * H * nb * nb * 4096);
+    return align_up((size_t)nbatch * H * nb * nb * 2048);
 }
 
 int kfh_bias_tiles_from_dense(const void* dense, int io_dtype, void* tiles, int nbatch, int H, int L,
@@ -100,7 +100,7 @@ int kfh_bias_tiles_from_dense(const void* dense, int io_dtype, void* tiles, int 
     if (!dense || !tiles || nbatch <= 0 || H <= 0 || L <= 0)
         return fail(KFH_EINVAL, "bias_tiles_from_dense: bad argument");
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "bias_tiles_from_dense: bad io_dtype %d", io_dtype);
-    launch_bias_tiles(dense, io_dtype, static_cast<float*>(tiles), nbatch, H, L, (L + 31) / 32,
+    launch_bias_tiles(dense, io_dtype, static_cast<uint16_t*>(tiles), nbatch, H, L, (L + 31) / 32,
                       static_cast<hipStream_t>(stream));
     return check_launch("bias_tiles_from_dense");
 }
@@ -132,10 +132,10 @@ int kfh_pair_bias_project(const void* z, const void* blob, void* tiles, int B, i
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const size_t nb = (N + 31) / 32, esz = io_dtype == KFH_F32 ? 4 : 2;
     for (int b = 0; b < B; ++b) {
-        float* t = static_cast<float*>(tiles) + (size_t)b * H * nb * nb * 1024;
+        uint16_t* t = static_cast<uint16_t*>(tiles) + (size_t)b * H * nb * nb * kBiasTileElems;
         if (N % 32) {   // queries beyond N in the last query block: keep their tiles finite
             for (int h = 0; h < H; ++h)
-                launch_fill_zero(t + (((size_t)h * nb + (nb - 1)) * nb) * 1024, nb * 4096, stream);
+                launch_fill_zero(t + (((size_t)h * nb + (nb - 1)) * nb) * kBiasTileElems, nb * 2048, stream);
         }
         launch_pair_bias(static_cast<const char*>(z) + (size_t)b * N * N * C * esz, io_dtype,
                          static_cast<const char*>(blob), t, N, H, eps, stream);
@@ -269,7 +269,7 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
     launch_key_codes(mask, codes, S, L, w.nb * 32, mask_per_sample ? L : 0, stream);
     FlashArgs fa{};
     fa.qf = ws + w.qf; fa.kf = ws + w.kf; fa.vf = ws + w.vf; fa.gf = ws + w.gf; fa.of = ws + w.of;
-    fa.biasf = bias_tiles; fa.codes = codes;
+    fa.biast = bias_tiles; fa.codes = codes;
     fa.nrows = S; fa.nb = w.nb; fa.H = H; fa.bias_per_row = bias_per_sample ? 1 : 0;
     if (launch_flash(fa, 32 * l.PB, stream) != 0) return fail(KFH_EUNSUPPORTED, "apb_forward: attention shape");
 

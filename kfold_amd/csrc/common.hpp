@@ -77,6 +77,15 @@ __device__ __forceinline__ void acc_to_frags(const f32x16& c, bf16x8& f0, bf16x8
     f1 = __builtin_bit_cast(bf16x8, b);
 }
 
+// Pair-bias tiles: a [32 queries x 32 keys] tile is stored as the two A-operand fragments of
+// bias^T (rows = keys, k = queries), bf16, 2 KiB: [k-step c][lane = key + 32*half][8], where
+// lane (key, half) of k-step c holds queries 16c + 8*half + 0..7.  The attention kernels add
+// the tile to the scores with two MFMAs against an identity B operand.
+constexpr int kBiasTileElems = 1024;
+__host__ __device__ __forceinline__ int bias_tile_elem(int q32, int k32) {
+    return (((q32 >> 4) * 64) + k32 + 32 * ((q32 >> 3) & 1)) * 8 + (q32 & 7);
+}
+
 // row index inside a 32x32 accumulator block for register v of this lane
 __device__ __forceinline__ int acc_row(int v, int half) { return 8 * (v >> 2) + 4 * half + (v & 3); }
 

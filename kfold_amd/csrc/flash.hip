@@ -11,178 +11,490 @@
 // All operands are in MFMA fragment order (see common.hpp):
 //   q, k, g, of : [row a][head h][block of 32 positions][k-step 0..DKS-1][lane][8 bf16]
 //   v           : [row a][head h][block of 32 keys][d-block 0..DV-1][k-step 0..1][lane][8 bf16]
-//   bias        : [bias batch][head h][query block][key block][4][lane][4 floats]
+//   bias        : [bias batch][head h][query block][key block] bf16 tiles of 2 KiB
 //   codes       : [row a][nb*32] bytes, 0 = beyond the sequence, 1 = masked key, 2 = valid key
 //
-// Wavefront = 32 queries of up to R rows for one head; workgroup = 4 adjacent query blocks.
-// S^T[key][query] = K Q^T + bias comes out of the MFMA with the bias tile as its C operand,
-// so a lane owns 16 keys of one query: the row max and row sum need one cross-half
-// exchange, and exp2(S - m) rounded to bf16 is already the B operand of
-// O^T[d][query] += V^T[d][key] P^T[key][query].  The R rows share the bias tile registers.
+// A wavefront computes S^T[key][query] for 32 keys x 32 queries with keys as accumulator rows:
+//   S^T = bias^T I + 1 (-m)^T + K Q^T
+// three MFMA groups into one accumulator: the bias tile against an identity operand, a
+// constant-one column against the running maximum m (so the accumulator is S - m and the
+// exponent needs no subtraction), and the scores.  A lane then owns 16 keys of one query: the
+// row max and row sum need one cross-half exchange, and exp2(S - m) rounded to bf16 is
+// already the B operand of O^T[d][query] += V^T[d][key] P^T[key][query].  m only moves when
+// a logit exceeds it by 2^8 (lazy rescale); it is kept bf16-representable so the MFMA
+// subtracts it exactly.
+//
+// Two kernels share that tile code:
+//   flash_strip_kernel  (triangle attention, N <= 1216): a workgroup owns one head, two query
+//       blocks and a range of rows; the bias strip of its query blocks (all key blocks) is
+//       loaded into LDS once, then each wavefront walks its rows with K/V fragments read
+//       straight from L2 — no barrier in the main loop, two score tiles in flight per step.
+//   flash_staged_kernel (any size / head dim): 8 wavefronts = 4 query blocks x 2 row groups;
+//       per key block K, V and bias tiles are staged in double-buffered LDS.
 //
 // Masking follows the reference's finite -1e9 semantics: in a row with a valid key, masked
 // keys get probability exactly 0; in a row with no valid key all real keys get the same
 // logit (q.k + bias is absorbed by -1e9 in fp32), i.e. uniform attention.
+#include <cstdlib>
+
 #include "kernels.hpp"
 
 namespace kfh {
 
-template <int R, int DKS, int DV>
-__global__ __launch_bounds__(256, (DKS == 2 ? 2 : 1)) void flash_kernel(FlashArgs p) {
-    static_assert(DKS == 2 * DV, "head dim = 16*DKS = 32*DV");
-    __shared__ uint8_t cls_s[4][R][256];      // per wavefront: class of each key block per row
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int half = lane >> 5;
-    const int nb = p.nb, H = p.H;
-    const bf16x8* __restrict__ qf = static_cast<const bf16x8*>(p.qf);
-    const bf16x8* __restrict__ kf = static_cast<const bf16x8*>(p.kf);
-    const bf16x8* __restrict__ vf = static_cast<const bf16x8*>(p.vf);
-    const bf16x8* __restrict__ gf = static_cast<const bf16x8*>(p.gf);
-    bf16x8* __restrict__ of = static_cast<bf16x8*>(p.of);
+constexpr float kLazyMax = 8.0f;   // rescale only when a logit exceeds the running max by 2^8
 
-    // chunk = (head, row set); all query groups of a chunk run on one XCD (workgroup ids are
-    // dealt round-robin over 8 XCDs); heads are the slowest index
+// bf16 fragment with one non-zero k-slot: slot 0 of the lanes with half == 0
+__device__ __forceinline__ bf16x8 slot0_frag(float v, int half) {
+    u32x4 w = {0u, 0u, 0u, 0u};
+    w[0] = half == 0 ? (pack_bf16(v, 0.f) & 0xffffu) : 0u;
+    return __builtin_bit_cast(bf16x8, w);
+}
+
+// identity B operand, k-step c: lane (col, half) holds I[j = 16c + 8*half + e][col]
+__device__ __forceinline__ bf16x8 identity_frag(int c, int col, int half) {
+    const int e = col - 16 * c - 8 * half;          // slot that holds the 1, if in 0..7
+    u32x4 w = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        if (e == 2 * i) w[i] = 0x00003f80u;
+        if (e == 2 * i + 1) w[i] = 0x3f800000u;
+    }
+    return __builtin_bit_cast(bf16x8, w);
+}
+
+__device__ __forceinline__ bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// Classify the key blocks of one row from its codes: 2 all valid, 1 some valid; with no valid
+// key: 0x82 all 32 keys real (masked), 0x81 some real, 0x80 none.  One wavefront; returns
+// true if the row has a valid key.
+__device__ __forceinline__ bool classify_row(const uint8_t* crow, int nb, int lane, uint8_t* cls) {
+    bool any_valid = false;
+    for (int base = 0; base < nb; base += 64) {
+        const int blk = base + lane;
+        int nvalid = 0, nreal = 0;
+        if (blk < nb) {
+            const u32x4* c = reinterpret_cast<const u32x4*>(crow + blk * 32);
+            const u32x4 c0 = c[0], c1 = c[1];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                nvalid += __popc(c0[i] & 0x02020202u) + __popc(c1[i] & 0x02020202u);
+                nreal += __popc(c0[i] & 0x03030303u) + __popc(c1[i] & 0x03030303u);
+            }
+            cls[blk] = nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal == 32 ? 0x82 : (nreal > 0 ? 0x81 : 0x80)));
+        }
+        const bool v = __ballot(nvalid > 0) != 0ull;
+        any_valid = any_valid || v;
+    }
+    return any_valid;
+}
+
+// mixed block: per-key select.  s holds S - m; this lane's keys are 8*(v/4) + 4*half + (v%4)
+__device__ __forceinline__ void mask_scores(f32x16& s, const uint8_t* codes_blk, int half, bool uni,
+                                            float m) {
+    const uint32_t* cw = reinterpret_cast<const uint32_t*>(codes_blk + 4 * half);
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        const uint32_t w = cw[2 * g];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t code = (w >> (8 * e)) & 0xffu;
+            const int v = 4 * g + e;
+            const float masked = (uni && code == 1) ? -m : -INFINITY;
+            s[v] = (!uni && code == 2) ? s[v] : masked;
+        }
+    }
+}
+
+__device__ __forceinline__ float tile_max(const f32x16& s) {
+    float mx = fmaxf(fmaxf(s[0], s[1]), s[2]);
+#pragma unroll
+    for (int v = 3; v < 15; v += 2) mx = fmaxf(fmaxf(mx, s[v]), s[v + 1]);
+    mx = fmaxf(mx, s[15]);
+    return xhalf_max(mx);
+}
+
+// move the running maximum by (bf16-rounded) mx and rescale the partial results
+template <int DV>
+__device__ __forceinline__ void rescale(f32x16& s, float mx, float& m, float& l, f32x16 (&o)[DV],
+                                        bf16x8& qx, int half) {
+    const float m_new = bf16_lo(pack_bf16(m + mx, 0.f));
+    const float delta = m_new - m;
+    const float alpha = fast_exp2(-delta);
+    m = m_new;
+    qx = slot0_frag(-m_new, half);
+    l *= alpha;
+#pragma unroll
+    for (int d = 0; d < DV; ++d)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) s[v] -= delta;
+}
+
+// Sum of 16 bf16 values held as 8 packed dwords: two chains of v_dot2c_f32_bf16 against a
+// vector of ones, fp32 accumulation.  Written as one inline-assembly block because (a) with
+// hipcc 7.2 the __builtin_amdgcn_fdot2_f32_bf16 form of this chain was compiled into four dot
+// products of the same source register, and (b) a DOT result needs three wait states before
+// a non-DOT VALU instruction may read it, which the compiler cannot know for inline
+// assembly: the trailing s_nop provides them.
+__device__ __forceinline__ float sum16_bf16(const u32x4& a, const u32x4& b) {
+    float t0 = 0.f, t1 = 0.f;
+    const uint32_t ones = 0x3f803f80u;
+    asm("v_dot2c_f32_bf16 %0, %2, %10\n\t"
+        "v_dot2c_f32_bf16 %1, %6, %10\n\t"
+        "v_dot2c_f32_bf16 %0, %3, %10\n\t"
+        "v_dot2c_f32_bf16 %1, %7, %10\n\t"
+        "v_dot2c_f32_bf16 %0, %4, %10\n\t"
+        "v_dot2c_f32_bf16 %1, %8, %10\n\t"
+        "v_dot2c_f32_bf16 %0, %5, %10\n\t"
+        "v_dot2c_f32_bf16 %1, %9, %10\n\t"
+        "s_nop 2"
+        : "+v"(t0), "+v"(t1)
+        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(ones));
+    return t0 + t1;
+}
+
+// p = bf16(exp2(s)) as the two B-operand fragments of the PV product; returns this lane's
+// partial row sum of the *rounded* probabilities, so the normaliser matches what the MFMA
+// accumulates.
+__device__ __forceinline__ float exp_pack_sum(const f32x16& s, bf16x8& p0, bf16x8& p1) {
+    u32x4 a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        a[i] = pack_bf16(fast_exp2(s[2 * i]), fast_exp2(s[2 * i + 1]));
+        b[i] = pack_bf16(fast_exp2(s[8 + 2 * i]), fast_exp2(s[8 + 2 * i + 1]));
+    }
+    p0 = __builtin_bit_cast(bf16x8, a);
+    p1 = __builtin_bit_cast(bf16x8, b);
+    return sum16_bf16(a, b);
+}
+
+// A lane's partial row sum above this (or inf / NaN from an overflowed exponent) sends the
+// tile through the exact max-and-rescale path instead.
+constexpr float kSumLimit = 1.0995116e12f;   // 2^40
+
+// ------------------------------------------------------------------------------------------
+// strip kernel (head dim 32)
+// ------------------------------------------------------------------------------------------
+constexpr int kStripWaves = 12;          // 768 threads, 3 wavefronts per SIMD, one workgroup per CU
+constexpr int kStripMaxBlocks = 38;      // 38 * 4 KiB strip + scratch <= 160 KiB LDS
+
+__global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashArgs p) {
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int nb = p.nb, H = p.H;
+    u32x4* strip = reinterpret_cast<u32x4*>(lds);                       // [kb][qbl][c][lane]
+    uint8_t* cls = reinterpret_cast<uint8_t*>(lds) + (size_t)nb * 4096 + wave * 64;
+    const u32x4* __restrict__ qf = static_cast<const u32x4*>(p.qf);
+    const u32x4* __restrict__ kf = static_cast<const u32x4*>(p.kf);
+    const u32x4* __restrict__ vf = static_cast<const u32x4*>(p.vf);
+    const u32x4* __restrict__ gf = static_cast<const u32x4*>(p.gf);
+    const u32x4* __restrict__ bt = static_cast<const u32x4*>(p.biast);
+    u32x4* __restrict__ of = static_cast<u32x4*>(p.of);
+
+    // chunk = (head, row range); the query-block pairs of a chunk share an XCD, heads slowest
     const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
     const int chunk = (slot / p.qgroups) * 8 + xcd;
     if (chunk >= p.nchunks) return;
-    const int qb = (slot % p.qgroups) * 4 + wave;
-    const int rowsets = (p.nrows + R - 1) / R;
-    const int h = chunk / rowsets, a0 = (chunk % rowsets) * R;
-    if (qb >= nb) return;
-    const int nr = min(R, p.nrows - a0);      // rows of this set that exist
+    const int pair = slot % p.qgroups;
+    const int h = chunk / p.rowranges, rr = chunk % p.rowranges;
+    const int qb[2] = {2 * pair, min(2 * pair + 1, nb - 1)};
+    const bool have_b = 2 * pair + 1 < nb;
 
-    auto qidx = [&](int a, int blk, int ks) -> size_t {
-        return ((((size_t)a * H + h) * nb + blk) * DKS + ks) * 64 + lane;
-    };
-    auto vidx = [&](int a, int blk, int d, int ks) -> size_t {
-        return (((((size_t)a * H + h) * nb + blk) * DV + d) * 2 + ks) * 64 + lane;
-    };
-
-    // ---- per row: classify key blocks: 2 all valid, 1 some valid, 0x81 real keys but none
-    // valid, 0x80 nothing --------------------------------------------------------------------
-    bool uniform_row[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) {
-        uniform_row[r] = false;
-        if (r >= nr) continue;
-        const uint8_t* crow = p.codes + (size_t)(a0 + r) * nb * 32;
-        bool any_valid = false;
-        for (int base = 0; base < nb; base += 64) {
-            const int blk = base + lane;
-            int nvalid = 0, nreal = 0;
-            if (blk < nb) {
-                const u32x4* c = reinterpret_cast<const u32x4*>(crow + blk * 32);
-                const u32x4 c0 = c[0], c1 = c[1];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    nvalid += __popc(c0[i] & 0x02020202u) + __popc(c1[i] & 0x02020202u);
-                    nreal += __popc(c0[i] & 0x03030303u) + __popc(c1[i] & 0x03030303u);
-                }
-                cls_s[wave][r][blk] = nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal > 0 ? 0x81 : 0x80));
-            }
-            const bool v = __ballot(nvalid > 0) != 0ull;
-            any_valid = any_valid || v;
-        }
-        uniform_row[r] = !any_valid;
+    // ---- bias strip of the two query blocks -> LDS -------------------------------------------
+    for (int u = tid; u < nb * 256; u += kStripWaves * 64) {
+        const int kb = u >> 8, qbl = (u >> 7) & 1, off = u & 127;
+        strip[u] = bt[(((size_t)h * nb + qb[qbl]) * nb + kb) * 128 + off];
     }
-    __builtin_amdgcn_s_waitcnt(0);   // the LDS bytes above are read back by this wavefront only
-    __builtin_amdgcn_wave_barrier();
+    __syncthreads();
 
-    bf16x8 q[R][DKS];
+    const bf16x8 kx = slot0_frag(1.0f, half);
+    const bf16x8 id0 = identity_frag(0, col, half), id1 = identity_frag(1, col, half);
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+    // rows are dealt round-robin over the row ranges so that every workgroup gets the same mix
+    // of padded and valid rows
+    for (int a = rr + p.rowranges * wave; a < p.nrows; a += p.rowranges * kStripWaves) {
+        const size_t row_units = ((size_t)a * H + h) * nb * 128;        // fragment units of (a, h)
+        const uint8_t* crow = p.codes + (size_t)a * nb * 32;
+        const bool uni = !classify_row(crow, nb, lane, cls);
+        bf16x8 q[2][2], qx[2];
+        f32x16 o[2][1];
+        float m[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            q[t][0] = as_frag(qf[row_units + qb[t] * 128 + lane]);
+            q[t][1] = as_frag(qf[row_units + qb[t] * 128 + 64 + lane]);
+            qx[t] = slot0_frag(0.f, half);
+            o[t][0] = zero;
+        }
+        bool first = true;
+        __builtin_amdgcn_s_waitcnt(0);   // cls bytes written above are read by this wavefront
+        __builtin_amdgcn_wave_barrier();
+
+        if (uni) {
+            // No valid key: every real key gets the same weight (see the masking note on top),
+            // whatever the query, so both query blocks get the plain sum of V over real keys.
+            const bf16x8 ones = as_frag(u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
+            for (int kb = 0; kb < nb; ++kb) {
+                const int c = __builtin_amdgcn_readfirstlane((int)cls[kb]);
+                if (c == 0x80) continue;
+                const u32x4* vp = vf + row_units + kb * 128 + lane;
+                const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
+                bf16x8 p0 = ones, p1 = ones;
+                float cnt = 16.f;
+                if (c != 0x82) {
+                    f32x16 sc = zero;
+                    mask_scores(sc, crow + kb * 32, half, true, 0.f);
+                    cnt = exp_pack_sum(sc, p0, p1);
+                }
+                l[0] += cnt;
+                o[0][0] = mfma32(v0, p0, o[0][0]);
+                o[0][0] = mfma32(v1, p1, o[0][0]);
+            }
+            l[1] = l[0];
+            o[1][0] = o[0][0];
+        } else
+        for (int kb = 0; kb < nb; ++kb) {
+            const int c = __builtin_amdgcn_readfirstlane((int)cls[kb]);
+            if (c & 0x80) continue;              // no valid key in this block
+            const u32x4* kp = kf + row_units + kb * 128 + lane;
+            const u32x4* vp = vf + row_units + kb * 128 + lane;
+            const bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
+            const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
+            const u32x4* sb = strip + kb * 256 + lane;
+            f32x16 s[2];
+            auto scores = [&]() {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    s[t] = mfma32(as_frag(sb[t * 128]), id0, zero);
+                    s[t] = mfma32(as_frag(sb[t * 128 + 64]), id1, s[t]);
+                    s[t] = mfma32(kx, qx[t], s[t]);
+                    s[t] = mfma32(k0, q[t][0], s[t]);
+                    s[t] = mfma32(k1, q[t][1], s[t]);
+                }
+            };
+            // exact path: mask, true maximum, rescale when it moved by more than 2^8
+            auto exact = [&]() {
+                if (c != 2) {
+                    mask_scores(s[0], crow + kb * 32, half, false, m[0]);
+                    mask_scores(s[1], crow + kb * 32, half, false, m[1]);
+                }
+                const float mx0 = tile_max(s[0]), mx1 = tile_max(s[1]);
+                if (first || __any(fmaxf(mx0, mx1) > kLazyMax)) {
+                    rescale<1>(s[0], mx0, m[0], l[0], o[0], qx[0], half);
+                    rescale<1>(s[1], mx1, m[1], l[1], o[1], qx[1], half);
+                }
+            };
+            scores();
+            if (first || c != 2) exact();
+            first = false;
+            // hot path: no maximum at all.  Scores of a row stay within range of its running
+            // maximum unless a later block towers over it; that shows up as a huge row sum.
+            bf16x8 p0[2], p1[2];
+            float ls0 = exp_pack_sum(s[0], p0[0], p1[0]);
+            float ls1 = exp_pack_sum(s[1], p0[1], p1[1]);
+            if (__any(!(fmaxf(ls0, ls1) < kSumLimit))) {
+                scores();
+                first = true;            // force the rescale in exact()
+                exact();
+                first = false;
+                ls0 = exp_pack_sum(s[0], p0[0], p1[0]);
+                ls1 = exp_pack_sum(s[1], p0[1], p1[1]);
+            }
+            l[0] += ls0;
+            l[1] += ls1;
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                o[t][0] = mfma32(v0, p0[t], o[t][0]);
+                o[t][0] = mfma32(v1, p1[t], o[t][0]);
+            }
+        }
+
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            if (t == 1 && !have_b) break;
+            const float inv = fast_rcp(xhalf_sum(l[t]));
+            const size_t u0 = row_units + qb[t] * 128 + lane;
+            const u32x4 g0 = gf[u0], g1 = gf[u0 + 64];
+            f32x16 og;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                og[2 * e] = o[t][0][2 * e] * inv * bf16_lo(g0[e]);
+                og[2 * e + 1] = o[t][0][2 * e + 1] * inv * bf16_hi(g0[e]);
+                og[8 + 2 * e] = o[t][0][8 + 2 * e] * inv * bf16_lo(g1[e]);
+                og[8 + 2 * e + 1] = o[t][0][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
+            }
+            bf16x8 f0, f1;
+            acc_to_frags(og, f0, f1);
+            of[u0] = __builtin_bit_cast(u32x4, f0);
+            of[u0 + 64] = __builtin_bit_cast(u32x4, f1);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// staged kernel (any sequence length, head dim 32 or 64)
+// ------------------------------------------------------------------------------------------
+template <int R, int DKS, int DV>
+__global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(FlashArgs p) {
+    static_assert(DKS == 2 * DV, "head dim = 16*DKS = 32*DV");
+    constexpr int A = 2 * R;                       // rows per workgroup
+    constexpr int KV_UNITS = DKS * 64;             // 16-byte units of one row's K (or V) block
+    constexpr int BIAS_OFF = 2 * A * KV_UNITS;     // unit offset of the bias tiles in a stage
+    constexpr int STAGE_UNITS = BIAS_OFF + 4 * 128;
+    constexpr int NLOAD = (STAGE_UNITS + 511) / 512;
+    __shared__ __attribute__((aligned(16))) u32x4 stage[2][STAGE_UNITS];
+    __shared__ uint8_t cls_s[A][256];              // class of each key block per row
+    __shared__ int uniform_s[A];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int nb = p.nb, H = p.H;
+    const u32x4* __restrict__ qf = static_cast<const u32x4*>(p.qf);
+    const u32x4* __restrict__ kf = static_cast<const u32x4*>(p.kf);
+    const u32x4* __restrict__ vf = static_cast<const u32x4*>(p.vf);
+    const u32x4* __restrict__ gf = static_cast<const u32x4*>(p.gf);
+    const u32x4* __restrict__ bt = static_cast<const u32x4*>(p.biast);
+    u32x4* __restrict__ of = static_cast<u32x4*>(p.of);
+
+    // chunk = (head, row set of A rows); the query groups of a chunk share an XCD
+    const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+    const int chunk = (slot / p.qgroups) * 8 + xcd;
+    if (chunk >= p.nchunks) return;
+    const int qb0 = (slot % p.qgroups) * 4;
+    const int rowsets = (p.nrows + A - 1) / A;
+    const int h = chunk / rowsets, a0 = (chunk % rowsets) * A;
+    const int qbl = wave & 3, rg = wave >> 2;      // this wavefront: query block, row group
+    const int qb = qb0 + qbl;
+    const bool wave_active = qb < nb;
+    const int qbc = min(qb, nb - 1);
+    const int nr = max(0, min(R, p.nrows - (a0 + rg * R)));   // rows of this wavefront that exist
+
+    auto rowc = [&](int ra) { return min(a0 + ra, p.nrows - 1); };                  // clamped row
+    auto blk_units = [&](int a, int blk) -> size_t {
+        return (((size_t)a * H + h) * nb + blk) * KV_UNITS;
+    };
+
+    if (wave < A) {
+        const bool any_valid = classify_row(p.codes + (size_t)rowc(wave) * nb * 32, nb, lane, cls_s[wave]);
+        if (lane == 0) uniform_s[wave] = any_valid ? 0 : 1;
+    }
+
+    u32x4 pre[NLOAD];
+    auto prefetch = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i) {
+            const int u = i * 512 + tid;
+            if (u < BIAS_OFF) {
+                const int region = u / KV_UNITS, off = u % KV_UNITS;      // K rows, then V rows
+                const u32x4* src = region < A ? kf : vf;
+                pre[i] = src[blk_units(rowc(region % A), kb) + off];
+            } else if (u < STAGE_UNITS) {
+                const int t = u - BIAS_OFF, q = t >> 7, off = t & 127;
+                pre[i] = bt[(((size_t)h * nb + min(qb0 + q, nb - 1)) * nb + kb) * 128 + off];
+            }
+        }
+    };
+    auto commit = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NLOAD; ++i) {
+            const int u = i * 512 + tid;
+            if (u < STAGE_UNITS) stage[buf][u] = pre[i];
+        }
+    };
+
+    const bf16x8 kx = slot0_frag(1.0f, half);
+    const bf16x8 id0 = identity_frag(0, col, half), id1 = identity_frag(1, col, half);
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    bf16x8 q[R][DKS], qx[R];
     f32x16 o[R][DV];
     float m[R], l[R];
+    bool first[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-        const int a = a0 + min(r, nr - 1);
+        const int a = rowc(rg * R + r);
 #pragma unroll
-        for (int ks = 0; ks < DKS; ++ks) q[r][ks] = qf[qidx(a, qb, ks)];
+        for (int ks = 0; ks < DKS; ++ks) q[r][ks] = as_frag(qf[blk_units(a, qbc) + ks * 64 + lane]);
+        qx[r] = slot0_frag(0.f, half);
 #pragma unroll
-        for (int d = 0; d < DV; ++d)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o[r][d][v] = 0.f;
-        m[r] = -1e30f;
+        for (int d = 0; d < DV; ++d) o[r][d] = zero;
+        m[r] = 0.f;
         l[r] = 0.f;
+        first[r] = true;
     }
 
-    const size_t bias_stride = (size_t)H * nb * nb * 256;     // f32x4 units per bias batch
+    prefetch(0);
+    commit(0);
+    __syncthreads();
+    bool uniform_row[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) uniform_row[r] = uniform_s[rg * R + r] != 0;
+
     for (int kb = 0; kb < nb; ++kb) {
-        f32x16 bias;
-        bool have_bias = false;
+        if (kb + 1 < nb) prefetch(kb + 1);
+        const u32x4* st = stage[kb & 1];
+        if (wave_active) {
+            const bf16x8 b0 = as_frag(st[BIAS_OFF + qbl * 128 + lane]);
+            const bf16x8 b1 = as_frag(st[BIAS_OFF + qbl * 128 + 64 + lane]);
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if (r >= nr) continue;
-            const int a = a0 + r;
-            int cls = __builtin_amdgcn_readfirstlane((int)cls_s[wave][r][kb]);
-            const bool uni = uniform_row[r];
-            if (cls & 0x80) {                    // no valid key in this block
-                if (!(uni && (cls & 1))) continue;
-                cls = 1;                         // uniform row: masked real keys take part
-            }
-            if (!have_bias || p.bias_per_row) {
-                const f32x4* bt = static_cast<const f32x4*>(p.biasf) +
-                                  (p.bias_per_row ? (size_t)a * bias_stride : 0) +
-                                  (((size_t)h * nb + qb) * nb + kb) * 256 + lane;
-                const f32x4 b0 = bt[0], b1 = bt[64], b2 = bt[128], b3 = bt[192];
+            for (int r = 0; r < R; ++r) {
+                if (r >= nr) continue;
+                const int ra = rg * R + r;
+                int cls = __builtin_amdgcn_readfirstlane((int)cls_s[ra][kb]);
+                const bool uni = uniform_row[r];
+                if (cls & 0x80) {                    // no valid key in this block
+                    if (!uni || cls == 0x80) continue;
+                    cls = 1;                         // uniform row: masked real keys take part
+                }
+                f32x16 s;
+                auto scores = [&]() {
+                    s = mfma32(b0, id0, zero);
+                    s = mfma32(b1, id1, s);
+                    s = mfma32(kx, qx[r], s);
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { bias[e] = b0[e]; bias[4 + e] = b1[e]; bias[8 + e] = b2[e]; bias[12 + e] = b3[e]; }
-                have_bias = true;
-            }
-            bf16x8 kk[DKS], vv[DV][2];
+                    for (int ks = 0; ks < DKS; ++ks)
+                        s = mfma32(as_frag(st[(ra * DKS + ks) * 64 + lane]), q[r][ks], s);
+                };
+                auto exact = [&](bool force) {
+                    if (cls != 2)
+                        mask_scores(s, p.codes + (size_t)(a0 + ra) * nb * 32 + kb * 32, half, uni, m[r]);
+                    const float mx = tile_max(s);
+                    if (force || __any(mx > kLazyMax)) rescale<DV>(s, mx, m[r], l[r], o[r], qx[r], half);
+                };
+                scores();
+                if (first[r] || cls != 2) exact(first[r]);
+                first[r] = false;
+                bf16x8 p0, p1;
+                float ls = exp_pack_sum(s, p0, p1);
+                if (__any(!(ls < kSumLimit))) {      // a block towering over the running maximum
+                    scores();
+                    exact(true);
+                    ls = exp_pack_sum(s, p0, p1);
+                }
+                l[r] += ls;
 #pragma unroll
-            for (int ks = 0; ks < DKS; ++ks) kk[ks] = kf[qidx(a, kb, ks)];
-#pragma unroll
-            for (int d = 0; d < DV; ++d) { vv[d][0] = vf[vidx(a, kb, d, 0)]; vv[d][1] = vf[vidx(a, kb, d, 1)]; }
-            f32x16 s = bias;
-#pragma unroll
-            for (int ks = 0; ks < DKS; ++ks) s = mfma32(kk[ks], q[r][ks], s);
-            if (cls != 2) {
-                // this lane's keys: 8*(v/4) + 4*half + (v%4) -> one dword of codes per 4 keys
-                const uint32_t* cw = reinterpret_cast<const uint32_t*>(
-                    p.codes + (size_t)a * nb * 32 + kb * 32 + 4 * half);
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    const uint32_t w = cw[2 * g];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint32_t code = (w >> (8 * e)) & 0xffu;
-                        const int v = 4 * g + e;
-                        if (uni) s[v] = code == 1 ? 0.f : -INFINITY;
-                        else if (code != 2) s[v] = -INFINITY;
-                    }
+                for (int d = 0; d < DV; ++d) {
+                    const u32x4* vt = st + A * KV_UNITS + (ra * DKS + 2 * d) * 64 + lane;
+                    o[r][d] = mfma32(as_frag(vt[0]), p0, o[r][d]);
+                    o[r][d] = mfma32(as_frag(vt[64]), p1, o[r][d]);
                 }
             }
-            float mx = s[0];
-#pragma unroll
-            for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
-            mx = xhalf_max(mx);
-            const float m_new = fmaxf(m[r], mx);
-            const float alpha = fast_exp2(m[r] - m_new);
-            m[r] = m_new;
-            float ls = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) { s[v] = fast_exp2(s[v] - m_new); ls += s[v]; }
-            l[r] = l[r] * alpha + ls;
-            bf16x8 p0, p1;
-            acc_to_frags(s, p0, p1);
-#pragma unroll
-            for (int d = 0; d < DV; ++d) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) o[r][d][v] *= alpha;
-                o[r][d] = mfma32(vv[d][0], p0, o[r][d]);
-                o[r][d] = mfma32(vv[d][1], p1, o[r][d]);
-            }
         }
+        if (kb + 1 < nb) commit((kb + 1) & 1);
+        __syncthreads();
     }
 
+    if (!wave_active) return;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (r >= nr) continue;
-        const int a = a0 + r;
+        const int a = a0 + rg * R + r;
         const float inv = fast_rcp(xhalf_sum(l[r]));
 #pragma unroll
         for (int d = 0; d < DV; ++d) {
-            const u32x4 g0 = __builtin_bit_cast(u32x4, gf[qidx(a, qb, 2 * d)]);
-            const u32x4 g1 = __builtin_bit_cast(u32x4, gf[qidx(a, qb, 2 * d + 1)]);
+            const size_t u0 = blk_units(a, qb) + (2 * d) * 64 + lane;
+            const u32x4 g0 = gf[u0], g1 = gf[u0 + 64];
             f32x16 og;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -193,26 +505,87 @@ __global__ __launch_bounds__(256, (DKS == 2 ? 2 : 1)) void flash_kernel(FlashArg
             }
             bf16x8 f0, f1;
             acc_to_frags(og, f0, f1);
-            of[qidx(a, qb, 2 * d)] = f0;
-            of[qidx(a, qb, 2 * d + 1)] = f1;
+            of[u0] = __builtin_bit_cast(u32x4, f0);
+            of[u0 + 64] = __builtin_bit_cast(u32x4, f1);
         }
     }
 }
 
-int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream) {
-    constexpr int R = 4;
-    FlashArgs p = args;
+static int launch_staged(FlashArgs p, int head_dim_pad, hipStream_t stream) {
+    constexpr int R = 1, A = 2 * R;
     p.qgroups = (p.nb + 3) / 4;
-    p.nchunks = p.H * ((p.nrows + R - 1) / R);
+    p.nchunks = p.H * ((p.nrows + A - 1) / A);
     const int nslots = ((p.nchunks + 7) / 8) * p.qgroups;
-    if (p.nb > 256) return -1;
     if (head_dim_pad == 32)
-        hipLaunchKernelGGL((flash_kernel<R, 2, 1>), dim3(nslots * 8), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((flash_staged_kernel<R, 2, 1>), dim3(nslots * 8), dim3(512), 0, stream, p);
     else if (head_dim_pad == 64)
-        hipLaunchKernelGGL((flash_kernel<R, 4, 2>), dim3(nslots * 8), dim3(256), 0, stream, p);
+        hipLaunchKernelGGL((flash_staged_kernel<R, 4, 2>), dim3(nslots * 8), dim3(512), 0, stream, p);
     else
         return -1;
     return 0;
+}
+
+static int launch_strip(FlashArgs p, hipStream_t stream) {
+    const size_t lds_bytes = (size_t)p.nb * 4096 + kStripWaves * 64;
+    static bool attr_set = false;
+    if (!attr_set) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_strip_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                kStripMaxBlocks * 4096 + kStripWaves * 64) != hipSuccess)
+            return -2;
+        attr_set = true;
+    }
+    p.qgroups = (p.nb + 1) / 2;                                    // query-block pairs
+    // rows per workgroup: a multiple of the wavefront count; one workgroup per CU is resident,
+    // so pick the split whose number of full-chip rounds times rows per round is smallest
+    static int n_cu = 0;
+    if (n_cu == 0) {
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0)
+            n_cu = 256;
+    }
+    int per = kStripWaves;
+    long long best = -1;
+    for (int cand = kStripWaves; cand <= kStripWaves * 8; cand += kStripWaves) {
+        const long long wgs = (long long)p.H * p.qgroups * ((p.nrows + cand - 1) / cand);
+        const long long cost = ((wgs + n_cu - 1) / n_cu) * cand;
+        if (best < 0 || cost <= best) { best = cost; per = cand; }
+    }
+    p.rows_per_range = per;
+    p.rowranges = (p.nrows + per - 1) / per;
+    p.nchunks = p.H * p.rowranges;
+    const int nslots = ((p.nchunks + 7) / 8) * p.qgroups;
+    hipLaunchKernelGGL(flash_strip_kernel, dim3(nslots * 8), dim3(kStripWaves * 64), lds_bytes, stream, p);
+    return 0;
+}
+
+int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream) {
+    if (args.nb > 256) return -1;
+    if (args.bias_per_row) {
+        // a workgroup stages one bias batch: run the rows one at a time
+        for (int a = 0; a < args.nrows; ++a) {
+            FlashArgs one = args;
+            const size_t frag_row = (size_t)args.H * args.nb * (head_dim_pad / 16) * 1024;
+            one.qf = static_cast<const char*>(args.qf) + a * frag_row;
+            one.kf = static_cast<const char*>(args.kf) + a * frag_row;
+            one.vf = static_cast<const char*>(args.vf) + a * frag_row;
+            one.gf = static_cast<const char*>(args.gf) + a * frag_row;
+            one.of = static_cast<char*>(args.of) + a * frag_row;
+            one.biast = static_cast<const char*>(args.biast) + (size_t)a * args.H * args.nb * args.nb * 2048;
+            one.codes = args.codes + (size_t)a * args.nb * 32;
+            one.nrows = 1;
+            one.bias_per_row = 0;
+            const int rc = launch_staged(one, head_dim_pad, stream);
+            if (rc) return rc;
+        }
+        return 0;
+    }
+    static const char* env = getenv("KFH_FLASH_STAGED");     // experiment knob
+    if (head_dim_pad == 32 && args.nb <= kStripMaxBlocks && args.nrows >= 4 * kStripWaves &&
+        !(env && env[0] == '1'))
+        return launch_strip(args, stream);
+    return launch_staged(args, head_dim_pad, stream);
 }
 
 }  // namespace kfh

@@ -55,7 +55,7 @@ constexpr size_t kTaBlobBytes = kTaLnOff + 2 * kC * sizeof(float);
 
 struct TriattnWorkspace {
     void *qf, *kf, *vf, *gf, *of;   // fragment buffers, N * 4 * nb * 2 KiB each
-    float* biasf;                    // 4 * nb * nb tiles of 4 KiB
+    uint16_t* biast;                 // 4 * nb * nb bf16 tiles of 2 KiB
     uint8_t* codes;                  // N * nb * 32 key codes
 };
 
@@ -63,11 +63,12 @@ struct TriattnWorkspace {
 struct FlashArgs {
     const void *qf, *kf, *vf, *gf;   // fragment-order operands
     void* of;                         // gated output fragments
-    const void* biasf;                // fp32 bias tiles
+    const void* biast;                // bf16 bias tiles (bias_tile_elem layout)
     const uint8_t* codes;             // [nrows][nb*32] key codes
     int nrows, nb, H;
     int bias_per_row;                 // 0: one bias for all rows, 1: bias batch index = row
     int qgroups, nchunks;             // filled in by launch_flash
+    int rowranges, rows_per_range;    // strip kernel: rows are split into ranges per workgroup
 };
 int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
 
@@ -88,7 +89,7 @@ int launch_pair_transition(const void* x, int io_dtype, const char* blob, int ex
 // ---- pair bias projection (pairbias.hip): blob = one packed block (heads as rows, scaled by
 // log2 e) followed by fp32 LN gamma, beta
 constexpr size_t kPbBlobBytes = kBlockBytes + 2 * kC * sizeof(float);
-void launch_pair_bias(const void* z, int io_dtype, const char* blob, float* tiles, int N, int H,
+void launch_pair_bias(const void* z, int io_dtype, const char* blob, uint16_t* tiles, int N, int H,
                       float eps, hipStream_t stream);
 
 // ---- single-track helpers (rows.hip, linear.hip) -------------------------------------------
@@ -96,7 +97,7 @@ int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const floa
                      long long M, int C, int normalize, float eps, hipStream_t stream);
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
                       long long mask_stride, hipStream_t stream);
-void launch_bias_tiles(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
+void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
                        hipStream_t stream);
 
 enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS };

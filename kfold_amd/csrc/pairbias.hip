@@ -1,7 +1,7 @@
 // Pair bias of the single-track attention:  bias[h, q, k] = (W LN(z[q, k]))[h]
 // (reference: model/modules/confidence_head.py:162-163, `linear_pair_bias(layernorm_z(z))`
 // moved to [B, H, L, L]).  One pass over z, HBM-bound on the z read; the result is written
-// directly as the log2(e)-scaled fp32 bias tiles the attention kernel consumes (flash.hip).
+// directly as the log2(e)-scaled bf16 bias tiles the attention kernels consume (flash.hip).
 #include "kernels.hpp"
 
 namespace kfh {
@@ -9,7 +9,7 @@ namespace kfh {
 template <int IO>
 __global__ __launch_bounds__(256) void pair_bias_kernel(const void* __restrict__ z,
                                                         const char* __restrict__ blob,
-                                                        float* __restrict__ tiles, int N, int nb,
+                                                        uint16_t* __restrict__ tiles, int N, int nb,
                                                         int H, float eps) {
     __shared__ __attribute__((aligned(16))) char smem[256 * kXS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void pair_bias_kernel(const void* __restrict__
             acc[pb] = mfma32(wk, lds_frag(smem, wave * 64 + 32 * pb + col, ks, half), acc[pb]);
     }
     // accumulator rows are heads; lane col is the key inside its block
-    const int lane_q = (a & 31) + 32 * ((col >> 2) & 1);
+    const int e = bias_tile_elem(a & 31, col);
 #pragma unroll
     for (int pb = 0; pb < 2; ++pb) {
         const int kblk = blk0 + pb;
@@ -46,13 +46,13 @@ __global__ __launch_bounds__(256) void pair_bias_kernel(const void* __restrict__
             const int h = acc_row(v, half);
             if (h < H) {
                 const size_t tile = ((size_t)h * nb + (a >> 5)) * nb + kblk;
-                tiles[((tile * 4 + (col >> 3)) * 64 + lane_q) * 4 + (col & 3)] = acc[pb][v];
+                tiles[tile * kBiasTileElems + e] = (uint16_t)(pack_bf16(acc[pb][v], 0.f) & 0xffffu);
             }
         }
     }
 }
 
-void launch_pair_bias(const void* z, int io_dtype, const char* blob, float* tiles, int N, int H,
+void launch_pair_bias(const void* z, int io_dtype, const char* blob, uint16_t* tiles, int N, int H,
                       float eps, hipStream_t stream) {
     const int nb = (N + 31) / 32;
     dim3 grid((N + 255) / 256, N), block(256);

@@ -92,30 +92,41 @@ void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int 
                        codes, rows, L, Lp, mask_stride);
 }
 
-// Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled fp32 tiles in accumulator order
-// [nbatch][H][qb][kb][group of 8 keys][lane = query + 32 * key-half][key % 4].
+// Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled bf16 tiles (bias_tile_elem layout);
+// one thread writes the 8 queries of one (tile, k-step, lane) slot.
 template <int IO>
-__global__ void bias_tiles_kernel(const void* __restrict__ dense, float* __restrict__ tiles,
+__global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __restrict__ tiles,
                                   long long total, int H, int L, int nb) {
-    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;      // 16-byte slot
     if (i >= total) return;
-    const int e = (int)(i & 3), lane = (int)((i >> 2) & 63), g = (int)((i >> 8) & 3);
-    long long t = i >> 10;
+    const int lane = (int)(i & 63), c = (int)((i >> 6) & 1);
+    long long t = i >> 7;
     const int kb = (int)(t % nb); t /= nb;
     const int qb = (int)(t % nb); t /= nb;          // t = batch * H + h
-    const int q = qb * 32 + (lane & 31), k = kb * 32 + 8 * g + 4 * (lane >> 5) + e;
-    float v = 0.f;
-    if (q < L && k < L) {
-        const size_t off = ((size_t)t * L + q) * L + k;
-        if constexpr (IO == KFH_F32) v = static_cast<const float*>(dense)[off];
-        else v = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
+    const int k = kb * 32 + (lane & 31);
+    uint32_t w[4];
+#pragma unroll
+    for (int e = 0; e < 8; e += 2) {
+        float v[2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            const int q = qb * 32 + 16 * c + 8 * (lane >> 5) + e + u;
+            float x = 0.f;
+            if (q < L && k < L) {
+                const size_t off = ((size_t)t * L + q) * L + k;
+                if constexpr (IO == KFH_F32) x = static_cast<const float*>(dense)[off];
+                else x = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
+            }
+            v[u] = x * kLog2e;
+        }
+        w[e >> 1] = pack_bf16(v[0], v[1]);
     }
-    tiles[i] = v * kLog2e;
+    reinterpret_cast<u32x4*>(tiles)[i] = u32x4{w[0], w[1], w[2], w[3]};
 }
 
-void launch_bias_tiles(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
+void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
                        hipStream_t stream) {
-    const long long total = (long long)nbatch * H * nb * nb * 1024;
+    const long long total = (long long)nbatch * H * nb * nb * 128;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, H, L, nb);

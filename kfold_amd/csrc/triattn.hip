@@ -37,7 +37,7 @@ template <int IO>
 __global__ __launch_bounds__(256) void triattn_proj_kernel(
     const void* __restrict__ x, const uint8_t* __restrict__ mask, const char* __restrict__ blob,
     bf16x8* __restrict__ qf, bf16x8* __restrict__ kf, bf16x8* __restrict__ vf,
-    bf16x8* __restrict__ gf, float* __restrict__ biasf, uint8_t* __restrict__ codes, int N, int nb,
+    bf16x8* __restrict__ gf, uint16_t* __restrict__ biast, uint8_t* __restrict__ codes, int N, int nb,
     int ending, float eps) {
     __shared__ __attribute__((aligned(16))) char smem[kTileA * kXS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -150,8 +150,8 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
 
     {
         // pair bias: x' position (a, b) is (query a, key b).  The heads are accumulator rows
-        // 0..3, i.e. registers v = 0..3 of the lanes with half == 0.  Scatter into the tile of
-        // (a/32, b/32) in accumulator order [group of 8 keys][lane = query + 32 * key-half][key % 4].
+        // 0..3, i.e. registers v = 0..3 of the lanes with half == 0.  Scatter into the bf16 tile
+        // of (a/32, b/32) (layout: bias_tile_elem in common.hpp).
         f32x16 acc[2];
 #pragma unroll
         for (int pb = 0; pb < 2; ++pb)
@@ -168,12 +168,11 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
             for (int pb = 0; pb < 2; ++pb) {
                 const int kblk = blk0 + pb;
                 if (kblk < nb) {
-                    const int kk = col;   // key index inside its block
-                    const int lane_q = (a & 31) + 32 * ((kk >> 2) & 1);
+                    const int e = bias_tile_elem(a & 31, col);   // lane col = key inside its block
 #pragma unroll
                     for (int h = 0; h < kH; ++h) {
                         const size_t tile = ((size_t)h * nb + (a >> 5)) * nb + kblk;
-                        biasf[((tile * 4 + (kk >> 3)) * 64 + lane_q) * 4 + (kk & 3)] = acc[pb][h];
+                        biast[tile * kBiasTileElems + e] = (uint16_t)(pack_bf16(acc[pb][h], 0.f) & 0xffffu);
                     }
                 }
             }
@@ -266,15 +265,15 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
     if (stages & KFH_STAGE_IN) {
         if (io_dtype == KFH_F32)
             hipLaunchKernelGGL(triattn_proj_kernel<KFH_F32>, grid_rows, block, 0, stream, x, mask, blob,
-                               qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+                               qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
         else
             hipLaunchKernelGGL(triattn_proj_kernel<KFH_BF16>, grid_rows, block, 0, stream, x, mask, blob,
-                               qf, kf, vf, gf, ws.biasf, ws.codes, N, nb, ending, eps);
+                               qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
     }
 
     FlashArgs fa{};
     fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = gf; fa.of = of;
-    fa.biasf = ws.biasf; fa.codes = ws.codes;
+    fa.biast = ws.biast; fa.codes = ws.codes;
     fa.nrows = N; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
     if (stages & KFH_STAGE_CORE) launch_flash(fa, 32, stream);
     if (!(stages & KFH_STAGE_OUT)) return;

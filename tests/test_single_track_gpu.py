@@ -90,15 +90,16 @@ def test_pair_bias_projection_and_trunk_apb(n):
                                   ref.linear_pair_bias.weight, device=torch.device(DEV))
         tiles = ops.pair_bias_project(zb.to(DEV), blob, 16)
         nb = (n + 31) // 32
-        t1 = tiles.view(torch.float32).view(16, nb, nb, 4, 64, 4)
-        t2 = tiles_dense.view(torch.float32).view(16, nb, nb, 4, 64, 4)
-        # compare only entries of real (query, key) pairs
-        q = (torch.arange(nb)[:, None] * 32 + torch.arange(64)[None, :] % 32)          # [qb, lane]
-        valid_q = (q < n)[None, :, None, None, :, None].to(DEV)
-        k = (torch.arange(nb)[:, None, None, None] * 32 + 8 * torch.arange(4)[None, :, None, None]
-             + 4 * (torch.arange(64)[None, None, :, None] // 32) + torch.arange(4)[None, None, None, :])
-        valid_k = (k < n)[None, None].to(DEV)
-        sel = (valid_q & valid_k).expand_as(t1)
+        # bf16 tiles [h][qb][kb][k-step c][lane = key + 32*half][e]; query = 16c + 8*half + e
+        t1 = tiles.view(torch.bfloat16).view(16, nb, nb, 2, 2, 32, 8).float()
+        t2 = tiles_dense.view(torch.bfloat16).view(16, nb, nb, 2, 2, 32, 8).float()
+        ar = torch.arange
+        q = (ar(nb)[:, None, None, None] * 32 + 16 * ar(2)[None, :, None, None]
+             + 8 * ar(2)[None, None, :, None] + ar(8)[None, None, None, :])            # [qb, c, half, e]
+        k = ar(nb)[:, None] * 32 + ar(32)[None, :]                                       # [kb, key]
+        valid_q = (q < n)[None, :, None, :, :, None, :]
+        valid_k = (k < n)[None, None, :, None, None, :, None]
+        sel = (valid_q & valid_k).expand_as(t1).to(DEV)
         assert_close(t1[sel], t2[sel], "pair bias tiles", max_abs=3e-2, mean_abs=3e-3, rel_fro=1e-2)
 
 
