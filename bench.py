@@ -201,7 +201,7 @@ def main() -> int:
         "block_mfma_frac": round(fl["block"] / ms_per_step / 1e9 / PEAK_BF16_TFLOPS, 4),
         "ops": ops_ms,
         "roofline": {
-            "kernel": "flash_kernel<4,2,1> (triangle attention, QK^T + softmax + PV)",
+            "kernel": "flash_strip_kernel (triangle attention, QK^T + softmax + PV)",
             "bound": "mfma",
             "achieved": round(achieved, 1),
             "peak": PEAK_BF16_TFLOPS,
