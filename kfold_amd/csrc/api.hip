@@ -35,11 +35,11 @@ int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w
     // input phase: step cb = { p_in rows 32cb.., g_in rows 32cb.. }
     for (int cb = 0; cb < 8; ++cb) {
         launch_pack_blocks(p_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, 1.f,
-                           b + kTmInOff + (2 * cb) * kBlockBytes, stream);
-        launch_pack_blocks(g_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, 1.f,
-                           b + kTmInOff + (2 * cb + 1) * kBlockBytes, stream);
+                           b + kTmAbOff + (2 * cb) * kBlockBytes, stream);
+        launch_pack_blocks(g_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, -kLog2e,
+                           b + kTmAbOff + (2 * cb + 1) * kBlockBytes, stream);
     }
-    launch_pack_blocks(g_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE2, K_NATURAL, 1.f,
+    launch_pack_blocks(g_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE2, K_NATURAL, -kLog2e,
                        b + kTmGateOff, stream);
     launch_pack_blocks(p_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE4, K_HALF, 1.f, b + kTmOutOff,
                        stream);

@@ -152,19 +152,20 @@ __device__ __forceinline__ u32x4 ln_row16(const float (&x)[8], const float (&gam
     return o;
 }
 
-// Stage ROWS LayerNorm-ed rows of 128 channels into an LDS tile (256 threads, 16 lanes per
-// row).  `row_off(row)` returns the element offset of the row in `src`, or -1 for a row
+// Stage ROWS LayerNorm-ed rows of 128 channels into an LDS tile (NTHREADS threads, 16 lanes
+// per row).  `row_off(row)` returns the element offset of the row in `src`, or -1 for a row
 // outside the tensor (staged as LN(0) = beta, finite).  `lnp` points at gamma[128], beta[128].
-template <int IO, int ROWS, class RowOff>
+template <int IO, int ROWS, class RowOff, int NTHREADS = 256>
 __device__ __forceinline__ void stage_ln_rows(char* tile, const void* src, const float* lnp,
                                               float eps, int tid, RowOff row_off) {
+    constexpr int RG = NTHREADS / 16;          // rows in flight per iteration
     const int r16 = tid >> 4, ch = tid & 15;
     float gam[8], bet[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) { gam[i] = lnp[ch * 8 + i]; bet[i] = lnp[kC + ch * 8 + i]; }
 #pragma unroll 2
-    for (int it = 0; it < ROWS / 16; ++it) {
-        const int row = it * 16 + r16;
+    for (int it = 0; it < ROWS / RG; ++it) {
+        const int row = it * RG + r16;
         const long long off = row_off(row);
         float x[8];
         if (off >= 0) {

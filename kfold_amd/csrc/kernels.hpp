@@ -19,12 +19,14 @@ void launch_copy_f32(const void* src, int wdtype, float* dst, int n, float fill,
 
 // ---- triangle multiplication (trimul.hip, contract.hip) ------------------------------------
 // Packed weight blob of one triangle-multiplication module (C = D = 128):
-//   [0, 128K)     8 steps x { p_in block cb, g_in block cb }   (32 channels of a|b each)
-//   [128K, 160K)  2 steps x { g_out blocks 2s, 2s+1 }          (ROW_INTERLEAVE2)
+//   [0, 32K)      2 steps x { g_out blocks 2s, 2s+1 }          (ROW_INTERLEAVE2)
+//   [32K, 160K)   8 steps x { p_in block cb, g_in block cb }   (32 channels of a|b each)
+//                 all gate weights (g_out, g_in) are pre-multiplied by -log2(e)
 //   [160K, 192K)  p_out, 4 blocks                               (ROW_INTERLEAVE4, K_HALF)
 //   [192K, +2K)   fp32: ln_in gamma, ln_in beta, ln_out gamma, ln_out beta (128 each)
-constexpr size_t kTmInOff = 0;
-constexpr size_t kTmGateOff = 16 * kBlockBytes;
+constexpr size_t kTmInOff = 0;                       // start of the 10 input-phase steps
+constexpr size_t kTmGateOff = 0;
+constexpr size_t kTmAbOff = 4 * kBlockBytes;
 constexpr size_t kTmOutOff = 20 * kBlockBytes;
 constexpr size_t kTmLnOff = 24 * kBlockBytes;
 constexpr size_t kTmBlobBytes = kTmLnOff + 4 * kC * sizeof(float);

@@ -33,8 +33,10 @@ __device__ __forceinline__ size_t frag_index(int a, int h, int blk, int ks, int 
 }
 
 // key codes: 0 = beyond N (padding of the last block), 1 = masked, 2 = valid
-template <int IO>
-__global__ __launch_bounds__(256) void triattn_proj_kernel(
+// PB = position blocks of 32 per wavefront: the workgroup has 8 / PB wavefronts.  PB = 1 keeps
+// the register count low enough for 4 wavefronts per SIMD.
+template <int IO, int PB>
+__global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kernel(
     const void* __restrict__ x, const uint8_t* __restrict__ mask, const char* __restrict__ blob,
     bf16x8* __restrict__ qf, bf16x8* __restrict__ kf, bf16x8* __restrict__ vf,
     bf16x8* __restrict__ gf, uint16_t* __restrict__ biast, uint8_t* __restrict__ codes, int N, int nb,
@@ -44,21 +46,23 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
     const int col = lane & 31, half = lane >> 5;
     const int a = blockIdx.y, t0 = blockIdx.x * kTileA;
 
-    stage_ln_rows<IO, kTileA>(smem, x, reinterpret_cast<const float*>(blob + kTaLnOff), eps, tid,
-                              [&](int row) -> long long {
-                                  const int b = t0 + row;
-                                  if (b >= N) return -1;
-                                  const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
-                                  return (long long)(pos * kC);
-                              });
+    constexpr int NT = 512 / PB;
+    auto row_off = [&](int row) -> long long {
+        const int b = t0 + row;
+        if (b >= N) return -1;
+        const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
+        return (long long)(pos * kC);
+    };
+    stage_ln_rows<IO, kTileA, decltype(row_off), NT>(
+        smem, x, reinterpret_cast<const float*>(blob + kTaLnOff), eps, tid, row_off);
     __syncthreads();
 
-    // wavefront = 64 positions = blocks blk0, blk0+1; lane col <-> position 32*pb + col
-    const int blk0 = (t0 + wave * 64) >> 5;
-    bf16x8 xf[2][kKS];
+    // wavefront = PB blocks of 32 positions starting at blk0; lane col <-> position 32*pb + col
+    const int blk0 = (t0 + wave * 32 * PB) >> 5;
+    bf16x8 xf[PB][kKS];
 #pragma unroll
-    for (int pb = 0; pb < 2; ++pb) {
-        const int row = wave * 64 + 32 * pb + col;
+    for (int pb = 0; pb < PB; ++pb) {
+        const int row = wave * 32 * PB + 32 * pb + col;
 #pragma unroll
         for (int ks = 0; ks < kKS; ++ks) xf[pb][ks] = lds_frag(smem, row, ks, half);
         const int b = t0 + row;
@@ -78,15 +82,16 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
     //   4..7  { g_h , v_h }   g_h like q; v_h with positions as rows (activations = A operand)
     //   8     { pair bias, - } rows 0..3 of the block are the 4 heads
     const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTaProjOff);
-    u32x4 pre[4];
+    constexpr int NPRE = 1024 / NT;
+    u32x4 pre[NPRE];
     auto prefetch = [&](int s) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) pre[i] = wsrc[s * 1024 + i * 256 + tid];
+        for (int i = 0; i < NPRE; ++i) pre[i] = wsrc[s * 1024 + i * NT + tid];
     };
     auto commit = [&](int s) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            reinterpret_cast<u32x4*>(smem + (s & 1) * 16384)[i * 256 + tid] = pre[i];
+        for (int i = 0; i < NPRE; ++i)
+            reinterpret_cast<u32x4*>(smem + (s & 1) * 16384)[i * NT + tid] = pre[i];
     };
     auto wfrag = [&](int s, int blk, int ks) {
         return *reinterpret_cast<const bf16x8*>(smem + (s & 1) * 16384 + blk * 8192 + ks * 1024 + lane * 16);
@@ -105,11 +110,11 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
         prefetch(s + 1);
         const bool gv = s >= 4;
         const int h = s & 3;
-        f32x16 acc[2][2];
+        f32x16 acc[2][PB];
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb)
+            for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[b][pb][v] = 0.f;
         if (!gv) {
@@ -117,7 +122,7 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
             for (int ks = 0; ks < kKS; ++ks) {
                 const bf16x8 w0 = wfrag(s, 0, ks), w1 = wfrag(s, 1, ks);
 #pragma unroll
-                for (int pb = 0; pb < 2; ++pb) {
+                for (int pb = 0; pb < PB; ++pb) {
                     acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
                     acc[1][pb] = mfma32(w1, xf[pb][ks], acc[1][pb]);
                 }
@@ -127,18 +132,18 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
             for (int ks = 0; ks < kKS; ++ks) {
                 const bf16x8 w0 = wfrag(s, 0, ks), w1 = wfrag(s, 1, ks);
 #pragma unroll
-                for (int pb = 0; pb < 2; ++pb) {
+                for (int pb = 0; pb < PB; ++pb) {
                     acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
                     acc[1][pb] = mfma32(xf[pb][ks], w1, acc[1][pb]);
                 }
             }
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb)
+            for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[0][pb][v] = sigmoidf_fast(acc[0][pb][v]);
         }
 #pragma unroll
-        for (int pb = 0; pb < 2; ++pb) {
+        for (int pb = 0; pb < PB; ++pb) {
             if (blk0 + pb < nb) {
                 store_frags(gv ? gf : qf, h, pb, acc[0][pb]);
                 store_frags(gv ? vf : kf, h, pb, acc[1][pb]);
@@ -152,20 +157,20 @@ __global__ __launch_bounds__(256) void triattn_proj_kernel(
         // pair bias: x' position (a, b) is (query a, key b).  The heads are accumulator rows
         // 0..3, i.e. registers v = 0..3 of the lanes with half == 0.  Scatter into the bf16 tile
         // of (a/32, b/32) (layout: bias_tile_elem in common.hpp).
-        f32x16 acc[2];
+        f32x16 acc[PB];
 #pragma unroll
-        for (int pb = 0; pb < 2; ++pb)
+        for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[pb][v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < kKS; ++ks) {
             const bf16x8 w0 = wfrag(8, 0, ks);
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb) acc[pb] = mfma32(w0, xf[pb][ks], acc[pb]);
+            for (int pb = 0; pb < PB; ++pb) acc[pb] = mfma32(w0, xf[pb][ks], acc[pb]);
         }
         if (half == 0) {
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb) {
+            for (int pb = 0; pb < PB; ++pb) {
                 const int kblk = blk0 + pb;
                 if (kblk < nb) {
                     const int e = bias_tile_elem(a & 31, col);   // lane col = key inside its block
@@ -264,11 +269,11 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
     dim3 grid_rows((N + kTileA - 1) / kTileA, N), block(256);
     if (stages & KFH_STAGE_IN) {
         if (io_dtype == KFH_F32)
-            hipLaunchKernelGGL(triattn_proj_kernel<KFH_F32>, grid_rows, block, 0, stream, x, mask, blob,
-                               qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
+            hipLaunchKernelGGL((triattn_proj_kernel<KFH_F32, 1>), grid_rows, dim3(512), 0, stream, x, mask,
+                               blob, qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
         else
-            hipLaunchKernelGGL(triattn_proj_kernel<KFH_BF16>, grid_rows, block, 0, stream, x, mask, blob,
-                               qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
+            hipLaunchKernelGGL((triattn_proj_kernel<KFH_BF16, 1>), grid_rows, dim3(512), 0, stream, x, mask,
+                               blob, qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
     }
 
     FlashArgs fa{};

@@ -18,133 +18,137 @@
 
 namespace kfh {
 
-constexpr int kTileP = 256;   // positions per workgroup in the input phase (64 per wavefront)
 
-template <int IO>
-__global__ __launch_bounds__(256) void trimul_in_kernel(
+// TILE positions per workgroup, 32 per wavefront: 32 fragment + 32 accumulator registers per
+// lane keep the kernel at 4 wavefronts per SIMD, which the VALU-heavy LayerNorm and gating
+// phases need; small tiles put several workgroups in different phases on one CU, so the
+// load phase of one overlaps the MFMA phase of another.
+template <int IO, int TILE>
+__global__ __launch_bounds__(TILE * 2, 4) void trimul_in_kernel(
     const void* __restrict__ z, const uint8_t* __restrict__ mask, const char* __restrict__ blob,
     uint16_t* __restrict__ planes, uint16_t* __restrict__ gate, int N, int Np, int incoming,
     float eps) {
     // staged LayerNorm rows first, then two 16 KiB weight buffers over the same memory
-    __shared__ __attribute__((aligned(16))) char smem[kTileP * kXS];
+    constexpr int NT = TILE * 2;
+    constexpr int SMEM = TILE * kXS > 32768 ? TILE * kXS : 32768;
+    __shared__ __attribute__((aligned(16))) char smem[SMEM];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
-    const int line = blockIdx.y, t0 = blockIdx.x * kTileP;
+    const int line = blockIdx.y, t0 = blockIdx.x * TILE;
     const size_t plane_sz = (size_t)Np * Np;
 
     if (line >= N) {   // padded line: zeros in every plane
-        const int t = t0 + 2 * (tid & 127);
+        const int t = t0 + 2 * (tid % (TILE / 2));
         if (t < Np) {
-            for (int ch = tid >> 7; ch < 2 * kC; ch += 2)
+            for (int ch = tid / (TILE / 2); ch < 2 * kC; ch += 4)
                 *reinterpret_cast<uint32_t*>(planes + ch * plane_sz + (size_t)line * Np + t) = 0u;
         }
         return;
     }
 
     // ---- phase A: load 256 rows, LayerNorm, stage as bf16 ---------------------------------
-    stage_ln_rows<IO, kTileP>(smem, z, reinterpret_cast<const float*>(blob + kTmLnOff), eps, tid,
-                              [&](int row) -> long long {
-                                  const int t = t0 + row;
-                                  if (t >= N) return -1;
-                                  const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
-                                  return (long long)(pos * kC);
-                              });
+    auto row_off = [&](int row) -> long long {
+        const int t = t0 + row;
+        if (t >= N) return -1;
+        const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
+        return (long long)(pos * kC);
+    };
+    stage_ln_rows<IO, TILE, decltype(row_off), NT>(
+        smem, z, reinterpret_cast<const float*>(blob + kTmLnOff), eps, tid, row_off);
     __syncthreads();
 
-    // ---- phase B: fragments of this wavefront's 64 positions; lane col <-> positions 2col+pb
-    bf16x8 xf[2][kKS];
-    float mk[2];
+    // ---- phase B: fragments of this wavefront's 32 positions; lane col <-> position 32*wave + col
+    const int tpos = t0 + wave * 32 + col;
+    bf16x8 xf[kKS];
 #pragma unroll
-    for (int pb = 0; pb < 2; ++pb) {
-        const int row = wave * 64 + 2 * col + pb, t = t0 + row;
-#pragma unroll
-        for (int ks = 0; ks < kKS; ++ks) xf[pb][ks] = lds_frag(smem, row, ks, half);
-        mk[pb] = 0.f;
-        if (t < N) {
-            const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
-            mk[pb] = mask[pos] ? 1.f : 0.f;
-        }
+    for (int ks = 0; ks < kKS; ++ks) xf[ks] = lds_frag(smem, wave * 32 + col, ks, half);
+    bool valid = false;
+    if (tpos < N) {
+        const size_t pos = incoming ? (size_t)tpos * N + line : (size_t)line * N + tpos;
+        valid = mask[pos] != 0;
     }
     __syncthreads();
 
-    // ---- phase C: 10 steps of two 32-column weight blocks, weights double-buffered in LDS --
+    // ---- phase C: 10 steps of two 32-column weight blocks (16 KiB), double-buffered in LDS:
+    //   0, 1   output-gate channels 64s + 2col + b   (activations = A operand, rows = positions)
+    //   2..9   a|b channels 32(s-2) .. +31: { p_in block, g_in block } (weights = A operand)
+    // Gate weights are packed pre-multiplied by -log2(e): sigmoid(g) = 1 / (1 + exp2(acc)).
+    // After the gate steps the fragments of masked positions are zeroed, which makes
+    // ab = p * sigmoid(g) * mask come out as exact zeros without a multiply (no bias terms).
     constexpr int NSTEP = 10;
     const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTmInOff);
-    u32x4 pre[4];
+    constexpr int NPRE = 1024 / NT;
+    u32x4 pre[NPRE];
+    auto prefetch = [&](int s) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) pre[i] = wsrc[i * 256 + tid];
+        for (int i = 0; i < NPRE; ++i) pre[i] = wsrc[s * 1024 + i * NT + tid];
+    };
+    auto commit = [&](int s) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) reinterpret_cast<u32x4*>(smem)[i * 256 + tid] = pre[i];
+        for (int i = 0; i < NPRE; ++i)
+            reinterpret_cast<u32x4*>(smem + (s & 1) * 16384)[i * NT + tid] = pre[i];
+    };
+    auto wfrag = [&](int s, int blk, int ks) {
+        return *reinterpret_cast<const bf16x8*>(smem + (s & 1) * 16384 + blk * 8192 + ks * 1024 + lane * 16);
+    };
+    prefetch(0);
+    commit(0);
     __syncthreads();
 
-    const int tpos = t0 + wave * 64 + 2 * col;
-    for (int s = 0; s < NSTEP; ++s) {
-        const char* wcur = smem + (s & 1) * 16384;
-        if (s + 1 < NSTEP) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i) pre[i] = wsrc[(s + 1) * 1024 + i * 256 + tid];
-        }
-        f32x16 acc[2][2];
+    for (int s = 0; s < 2; ++s) {
+        prefetch(s + 1);
+        f32x16 acc[2];
 #pragma unroll
         for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb)
+            for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[b][pb][v] = 0.f;
+        for (int ks = 0; ks < kKS; ++ks) {
+            acc[0] = mfma32(xf[ks], wfrag(s, 0, ks), acc[0]);
+            acc[1] = mfma32(xf[ks], wfrag(s, 1, ks), acc[1]);
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int t = t0 + wave * 32 + acc_row(v, half);
+            if (t < N) {
+                const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
+                *reinterpret_cast<uint32_t*>(gate + pos * kC + 64 * s + 2 * col) =
+                    pack_bf16(fast_rcp(1.0f + fast_exp2(acc[0][v])), fast_rcp(1.0f + fast_exp2(acc[1][v])));
+            }
+        }
+        commit(s + 1);
+        __syncthreads();
+    }
 
-        if (s < 8) {
-            // a|b channels 32s..32s+31: weights as the A operand (rows = channels)
 #pragma unroll
-            for (int ks = 0; ks < kKS; ++ks) {
-                const bf16x8 w0 = *reinterpret_cast<const bf16x8*>(wcur + ks * 1024 + lane * 16);
-                const bf16x8 w1 = *reinterpret_cast<const bf16x8*>(wcur + 8192 + ks * 1024 + lane * 16);
+    for (int ks = 0; ks < kKS; ++ks) {
+        u32x4 w = __builtin_bit_cast(u32x4, xf[ks]);
 #pragma unroll
-                for (int pb = 0; pb < 2; ++pb) {
-                    acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
-                    acc[1][pb] = mfma32(w1, xf[pb][ks], acc[1][pb]);
-                }
-            }
-            if (tpos < Np) {
+        for (int i = 0; i < 4; ++i) w[i] = valid ? w[i] : 0u;
+        xf[ks] = __builtin_bit_cast(bf16x8, w);
+    }
+
+    for (int s = 2; s < NSTEP; ++s) {
+        if (s + 1 < NSTEP) prefetch(s + 1);
+        f32x16 acc[2];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int chn = s * 32 + acc_row(v, half);
-                    const float a0 = acc[0][0][v] * sigmoidf_fast(acc[1][0][v]) * mk[0];
-                    const float a1 = acc[0][1][v] * sigmoidf_fast(acc[1][1][v]) * mk[1];
-                    *reinterpret_cast<uint32_t*>(planes + chn * plane_sz + (size_t)line * Np + tpos) =
-                        pack_bf16(a0, a1);
-                }
-            }
-        } else {
-            // output gate channels 64gs + 2col + b: activations as the A operand (rows = positions)
-            const int gs = s - 8;
+        for (int b = 0; b < 2; ++b)
 #pragma unroll
-            for (int ks = 0; ks < kKS; ++ks) {
-                const bf16x8 w0 = *reinterpret_cast<const bf16x8*>(wcur + ks * 1024 + lane * 16);
-                const bf16x8 w1 = *reinterpret_cast<const bf16x8*>(wcur + 8192 + ks * 1024 + lane * 16);
+            for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
 #pragma unroll
-                for (int pb = 0; pb < 2; ++pb) {
-                    acc[0][pb] = mfma32(xf[pb][ks], w0, acc[0][pb]);
-                    acc[1][pb] = mfma32(xf[pb][ks], w1, acc[1][pb]);
-                }
-            }
+        for (int ks = 0; ks < kKS; ++ks) {
+            acc[0] = mfma32(wfrag(s, 0, ks), xf[ks], acc[0]);
+            acc[1] = mfma32(wfrag(s, 1, ks), xf[ks], acc[1]);
+        }
+        if (tpos < Np) {
+            uint16_t* dst = planes + (size_t)((s - 2) * 32) * plane_sz + (size_t)line * Np + tpos;
 #pragma unroll
-            for (int pb = 0; pb < 2; ++pb) {
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int t = t0 + wave * 64 + 2 * acc_row(v, half) + pb;
-                    if (t < N) {
-                        const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
-                        *reinterpret_cast<uint32_t*>(gate + pos * kC + 64 * gs + 2 * col) =
-                            pack_bf16(sigmoidf_fast(acc[0][pb][v]), sigmoidf_fast(acc[1][pb][v]));
-                    }
-                }
+            for (int v = 0; v < 16; ++v) {
+                const float a0 = acc[0][v] * fast_rcp(1.0f + fast_exp2(acc[1][v]));
+                dst[(size_t)acc_row(v, half) * plane_sz] = (uint16_t)(pack_bf16(a0, 0.f) & 0xffffu);
             }
         }
-        if (s + 1 < NSTEP) {
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-                reinterpret_cast<u32x4*>(smem + ((s + 1) & 1) * 16384)[i * 256 + tid] = pre[i];
-        }
+        if (s + 1 < NSTEP) commit(s + 1);
         __syncthreads();
     }
 }
@@ -152,13 +156,14 @@ __global__ __launch_bounds__(256) void trimul_in_kernel(
 void launch_trimul_in(const void* z, int io_dtype, const uint8_t* mask, const char* blob,
                       uint16_t* planes, uint16_t* gate, int N, int Np, int incoming, float eps,
                       hipStream_t stream) {
-    dim3 grid((Np + kTileP - 1) / kTileP, Np), block(256);
+    constexpr int TILE = 256;
+    dim3 grid((Np + TILE - 1) / TILE, Np), block(TILE * 2);
     if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(trimul_in_kernel<KFH_F32>, grid, block, 0, stream, z, mask, blob, planes,
+        hipLaunchKernelGGL((trimul_in_kernel<KFH_F32, TILE>), grid, block, 0, stream, z, mask, blob, planes,
                            gate, N, Np, incoming, eps);
     else
-        hipLaunchKernelGGL(trimul_in_kernel<KFH_BF16>, grid, block, 0, stream, z, mask, blob, planes,
-                           gate, N, Np, incoming, eps);
+        hipLaunchKernelGGL((trimul_in_kernel<KFH_BF16, TILE>), grid, block, 0, stream, z, mask, blob,
+                           planes, gate, N, Np, incoming, eps);
 }
 
 // -----------------------------------------------------------------------------------------
