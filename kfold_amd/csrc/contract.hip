@@ -4,8 +4,8 @@
 // input phase has laid a and b out channel-major; planes are Np x Np, zero padded).
 //
 // Workgroup = 4 wavefronts in a 2x2 grid, each owning WM x WN accumulator blocks of 32x32.
-// K is walked in tiles of 32 through double-buffered LDS; the next tile's global loads are
-// issued before the current tile's MFMAs.  Rows of the B tile are stored to LDS permuted
+// K is walked in tiles of BK through double-buffered LDS with a third tile in flight in
+// registers.  Rows of the B tile are stored to LDS permuted
 // (row WN*c + n of a wavefront's range goes to block n, column c) so that after the MFMA a
 // lane owns WN adjacent output columns and writes them with one store.
 //
@@ -13,16 +13,35 @@
 // ids are dealt round-robin over the 8 XCDs): the two planes of a channel are then read
 // from HBM once and served from that XCD's L2 afterwards.
 #include "kernels.hpp"
+#include <cstdlib>
 
 namespace kfh {
 
-template <int WM, int WN>
-__global__ __launch_bounds__(256) void contract_kernel(const uint16_t* __restrict__ A,
+template <int MASK, int N, int SYNC>
+__device__ __forceinline__ void sched_group() {
+    if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, SYNC);
+}
+
+// Instruction order of one k-step: NM MFMAs (mask 0x008) with the NFR fragment reads (0x100)
+// and NLD operations of kind EXTRA (0x200 LDS stores, 0x020 global loads, 0 none) spread
+// evenly between them.
+template <int I, int NM, int NFR, int NLD, int EXTRA, int SYNC>
+__device__ __forceinline__ void schedule_kstep() {
+    if constexpr (I < NM) {
+        sched_group<0x100, ((I + 1) * NFR) / NM - (I * NFR) / NM, SYNC>();
+        if constexpr (EXTRA != 0) sched_group<EXTRA, ((I + 1) * NLD) / NM - (I * NLD) / NM, SYNC>();
+        sched_group<0x008, 1, SYNC>();
+        schedule_kstep<I + 1, NM, NFR, NLD, EXTRA, SYNC>();
+    }
+}
+
+template <int WM, int WN, int BK, int OCC>
+__global__ __launch_bounds__(256, OCC) void contract_kernel(const uint16_t* __restrict__ A,
                                                        const uint16_t* __restrict__ B,
                                                        uint16_t* __restrict__ Y, int Np,
                                                        int tiles_m, int tiles_n) {
-    constexpr int BM = 64 * WM, BN = 64 * WN, BK = 32;
-    constexpr int RS = 80;                  // bytes per LDS row: 32 bf16 + 16 B padding
+    constexpr int BM = 64 * WM, BN = 64 * WN;
+    constexpr int RS = BK * 2 + 16;         // bytes per LDS row: BK bf16 + 16 B padding
     constexpr int SKEW = 64;                // extra bytes per 32-row group of the B tile
     constexpr int A_BYTES = BM * RS;
     constexpr int B_BYTES = BN * RS + (BN / 32) * SKEW;
@@ -41,14 +60,16 @@ __global__ __launch_bounds__(256) void contract_kernel(const uint16_t* __restric
     const uint16_t* Ad = A + (size_t)d * Np * Np + (size_t)tm * BM * Np;
     const uint16_t* Bd = B + (size_t)d * Np * Np + (size_t)tn * BN * Np;
 
-    constexpr int ITA = BM / 64, ITB = BN / 64;
-    const int lrow = tid >> 2, lchunk = tid & 3;
+    constexpr int CPR = BK / 8;             // 16-byte chunks per tile row
+    constexpr int RPP = 256 / CPR;          // rows per pass of the 256 threads
+    constexpr int ITA = BM / RPP, ITB = BN / RPP;
+    const int lrow = tid / CPR, lchunk = tid % CPR;
     u32x4 ra[ITA], rb[ITB];
     // LDS byte offset of B-tile row g (0..BN-1) after the column permutation
     int boff[ITB];
 #pragma unroll
     for (int it = 0; it < ITB; ++it) {
-        const int g = lrow + 64 * it;
+        const int g = lrow + RPP * it;
         const int w = g / (32 * WN), gl = g % (32 * WN);
         const int blk = w * WN + gl % WN;             // 32-row group in LDS
         boff[it] = (blk * 32 + gl / WN) * RS + blk * SKEW + lchunk * 16;
@@ -57,17 +78,17 @@ __global__ __launch_bounds__(256) void contract_kernel(const uint16_t* __restric
     auto gload = [&](int kt) {
 #pragma unroll
         for (int it = 0; it < ITA; ++it)
-            ra[it] = *reinterpret_cast<const u32x4*>(Ad + (size_t)(lrow + 64 * it) * Np + kt * BK + lchunk * 8);
+            ra[it] = *reinterpret_cast<const u32x4*>(Ad + (size_t)(lrow + RPP * it) * Np + kt * BK + lchunk * 8);
 #pragma unroll
         for (int it = 0; it < ITB; ++it)
-            rb[it] = *reinterpret_cast<const u32x4*>(Bd + (size_t)(lrow + 64 * it) * Np + kt * BK + lchunk * 8);
+            rb[it] = *reinterpret_cast<const u32x4*>(Bd + (size_t)(lrow + RPP * it) * Np + kt * BK + lchunk * 8);
     };
     auto lstore = [&](int buf) {
         char* as = lds + buf * (A_BYTES + B_BYTES);
         char* bs = as + A_BYTES;
 #pragma unroll
         for (int it = 0; it < ITA; ++it)
-            *reinterpret_cast<u32x4*>(as + (lrow + 64 * it) * RS + lchunk * 16) = ra[it];
+            *reinterpret_cast<u32x4*>(as + (lrow + RPP * it) * RS + lchunk * 16) = ra[it];
 #pragma unroll
         for (int it = 0; it < ITB; ++it) *reinterpret_cast<u32x4*>(bs + boff[it]) = rb[it];
     };
@@ -80,33 +101,70 @@ __global__ __launch_bounds__(256) void contract_kernel(const uint16_t* __restric
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[m][n][v] = 0.f;
 
+    constexpr int KS = BK / 16;             // MFMA k-steps per tile
+    constexpr int NFR = WM + WN;            // fragment reads per k-step
+    constexpr int NM = WM * WN;             // MFMAs per k-step
+    constexpr int NLD = ITA + ITB;          // tile loads (and LDS stores) per thread
+    static_assert(KS == 2 || KS == 4, "schedule shape");
+
+    bf16x8 af[2][WM], bf[2][WN];
+    auto load_frags = [&](int buf, int ks, int slot) {
+        const char* as = lds + buf * (A_BYTES + B_BYTES);
+        const char* bs = as + A_BYTES;
+#pragma unroll
+        for (int m = 0; m < WM; ++m)
+            af[slot][m] = *reinterpret_cast<const bf16x8*>(as + ((wm * WM + m) * 32 + col) * RS + ks * 32 + half * 16);
+#pragma unroll
+        for (int n = 0; n < WN; ++n) {
+            const int blk = wn * WN + n;
+            bf[slot][n] = *reinterpret_cast<const bf16x8*>(bs + (blk * 32 + col) * RS + blk * SKEW + ks * 32 + half * 16);
+        }
+    };
+    auto mfmas = [&](int slot) {
+#pragma unroll
+        for (int m = 0; m < WM; ++m)
+#pragma unroll
+            for (int n = 0; n < WN; ++n) acc[m][n] = mfma32(af[slot][m], bf[slot][n], acc[m][n]);
+    };
+
+    // Software pipeline, one branch-free body per tile kt:
+    //   registers -> LDS for tile kt+1, global -> registers for tile kt+2, and the fragments of
+    //   k-step ks+1 are read from LDS while the MFMAs of k-step ks run.  The single barrier sits
+    //   before the last k-step, whose MFMAs cover the first fragment reads of tile kt+1.
+    // Tile indices past the end are clamped: the surplus loads and stores touch valid memory
+    // that nothing reads afterwards.
     const int KT = Np / BK;
     gload(0);
     lstore(0);
+    gload(KT > 1 ? 1 : 0);
     __syncthreads();
+    load_frags(0, 0, 0);
     for (int kt = 0; kt < KT; ++kt) {
         const int cur = kt & 1;
-        if (kt + 1 < KT) gload(kt + 1);
-        const char* as = lds + cur * (A_BYTES + B_BYTES);
-        const char* bs = as + A_BYTES;
-#pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            bf16x8 af[WM], bf[WN];
-#pragma unroll
-            for (int m = 0; m < WM; ++m)
-                af[m] = *reinterpret_cast<const bf16x8*>(as + ((wm * WM + m) * 32 + col) * RS + ks * 32 + half * 16);
-#pragma unroll
-            for (int n = 0; n < WN; ++n) {
-                const int blk = wn * WN + n;
-                bf[n] = *reinterpret_cast<const bf16x8*>(bs + (blk * 32 + col) * RS + blk * SKEW + ks * 32 + half * 16);
-            }
-#pragma unroll
-            for (int m = 0; m < WM; ++m)
-#pragma unroll
-                for (int n = 0; n < WN; ++n) acc[m][n] = mfma32(af[m], bf[n], acc[m][n]);
+        lstore(cur ^ 1);
+        gload(kt + 2 < KT ? kt + 2 : KT - 1);
+        if constexpr (KS == 4) {
+            load_frags(cur, 1, 1);
+            mfmas(0);
+            load_frags(cur, 2, 0);
+            mfmas(1);
+            load_frags(cur, 3, 1);
+            mfmas(0);
+            schedule_kstep<0, NM, NFR, NLD, 0x200, 0>();      // + LDS tile stores
+            schedule_kstep<0, NM, NFR, NLD, 0x020, 0>();      // + global tile loads
+            schedule_kstep<0, NM, NFR, NLD, 0, 0>();
+        } else {
+            load_frags(cur, 1, 1);
+            mfmas(0);
+            schedule_kstep<0, NM, NFR, NLD, 0x200, 0>();
         }
-        if (kt + 1 < KT) lstore(cur ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        load_frags(cur ^ 1, 0, 0);
+        mfmas(1);
+        if constexpr (KS == 4) schedule_kstep<0, NM, NFR, NLD, 0, 1>();
+        else schedule_kstep<0, NM, NFR, NLD, 0x020, 1>();
     }
 
     // lane (col, half) owns rows acc_row(v, half) and the WN adjacent columns WN*col + n
@@ -132,13 +190,22 @@ __global__ __launch_bounds__(256) void contract_kernel(const uint16_t* __restric
 void launch_contract(const uint16_t* planes_a, const uint16_t* planes_b, uint16_t* planes_y,
                      int Np, int D, hipStream_t stream) {
     // Np is a multiple of 128; use 256x256 tiles when they divide it, else 128x128
-    if (Np % 256 == 0) {
+    static const int variant = getenv("KFH_CONTRACT") ? atoi(getenv("KFH_CONTRACT")) : 0;
+    if (Np % 256 == 0 && variant == 0) {
         const int t = Np / 256;
-        hipLaunchKernelGGL((contract_kernel<4, 4>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
+        hipLaunchKernelGGL((contract_kernel<4, 4, 64, 1>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
                            planes_b, planes_y, Np, t, t);
+    } else if (Np % 256 == 0 && variant == 1) {
+        const int tm = Np / 256, tn = Np / 128;
+        hipLaunchKernelGGL((contract_kernel<4, 2, 32, 2>), dim3(D * tm * tn), dim3(256), 0, stream, planes_a,
+                           planes_b, planes_y, Np, tm, tn);
+    } else if (Np % 256 == 0 && variant == 2) {
+        const int tm = Np / 128, tn = Np / 256;
+        hipLaunchKernelGGL((contract_kernel<2, 4, 32, 2>), dim3(D * tm * tn), dim3(256), 0, stream, planes_a,
+                           planes_b, planes_y, Np, tm, tn);
     } else {
         const int t = Np / 128;
-        hipLaunchKernelGGL((contract_kernel<2, 2>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
+        hipLaunchKernelGGL((contract_kernel<2, 2, 64, 2>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
                            planes_b, planes_y, Np, t, t);
     }
 }
