@@ -77,13 +77,27 @@ __device__ __forceinline__ void acc_to_frags(const f32x16& c, bf16x8& f0, bf16x8
     f1 = __builtin_bit_cast(bf16x8, b);
 }
 
-// Pair-bias tiles: a [32 queries x 32 keys] tile is stored as the two A-operand fragments of
-// bias^T (rows = keys, k = queries), bf16, 2 KiB: [k-step c][lane = key + 32*half][8], where
-// lane (key, half) of k-step c holds queries 16c + 8*half + 0..7.  The attention kernels add
-// the tile to the scores with two MFMAs against an identity B operand.
+// Pair-bias tiles: a [32 queries x 32 keys] tile is stored in bf16 (2 KiB) in the register
+// order of the transposed score accumulator S^T[key][query]: [chunk c][lane = query + 32*half][8],
+// where element j of chunk c is accumulator register v = 8c + j, i.e. key
+// 8*(v/4) + 4*half + v%4.  The attention kernels read a tile with two 16-byte loads per lane
+// and widen it to the fp32 C operand of the first score MFMA.
 constexpr int kBiasTileElems = 1024;
 __host__ __device__ __forceinline__ int bias_tile_elem(int q32, int k32) {
-    return (((q32 >> 4) * 64) + k32 + 32 * ((q32 >> 3) & 1)) * 8 + (q32 & 7);
+    const int v = 4 * (k32 >> 3) + (k32 & 3), lane = q32 + 32 * ((k32 >> 2) & 1);
+    return ((v >> 3) * 64 + lane) * 8 + (v & 7);
+}
+// the two 16-byte chunks of a tile held by this lane -> fp32 accumulator registers
+__device__ __forceinline__ f32x16 bias_tile_acc(const u32x4& c0, const u32x4& c1) {
+    f32x16 r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        r[2 * i] = __uint_as_float(c0[i] << 16);
+        r[2 * i + 1] = __uint_as_float(c0[i] & 0xffff0000u);
+        r[8 + 2 * i] = __uint_as_float(c1[i] << 16);
+        r[8 + 2 * i + 1] = __uint_as_float(c1[i] & 0xffff0000u);
+    }
+    return r;
 }
 
 // row index inside a 32x32 accumulator block for register v of this lane

@@ -15,10 +15,10 @@
 //   codes       : [row a][nb*32] bytes, 0 = beyond the sequence, 1 = masked key, 2 = valid key
 //
 // A wavefront computes S^T[key][query] for 32 keys x 32 queries with keys as accumulator rows:
-//   S^T = bias^T I + 1 (-m)^T + K Q^T
-// three MFMA groups into one accumulator: the bias tile against an identity operand, a
-// constant-one column against the running maximum m (so the accumulator is S - m and the
-// exponent needs no subtraction), and the scores.  A lane then owns 16 keys of one query: the
+//   S^T = bias^T + 1 (-m)^T + K Q^T
+// the bias tile (stored in accumulator register order, widened from bf16) is the C operand, a
+// constant-one column against the running maximum m makes the accumulator S - m (so the
+// exponent needs no subtraction), then the scores.  A lane then owns 16 keys of one query: the
 // row max and row sum need one cross-half exchange, and exp2(S - m) rounded to bf16 is
 // already the B operand of O^T[d][query] += V^T[d][key] P^T[key][query].  m only moves when
 // a logit exceeds it by 2^8 (lazy rescale); it is kept bf16-representable so the MFMA
@@ -50,24 +50,13 @@ __device__ __forceinline__ bf16x8 slot0_frag(float v, int half) {
     return __builtin_bit_cast(bf16x8, w);
 }
 
-// identity B operand, k-step c: lane (col, half) holds I[j = 16c + 8*half + e][col]
-__device__ __forceinline__ bf16x8 identity_frag(int c, int col, int half) {
-    const int e = col - 16 * c - 8 * half;          // slot that holds the 1, if in 0..7
-    u32x4 w = {0u, 0u, 0u, 0u};
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        if (e == 2 * i) w[i] = 0x00003f80u;
-        if (e == 2 * i + 1) w[i] = 0x3f800000u;
-    }
-    return __builtin_bit_cast(bf16x8, w);
-}
-
 __device__ __forceinline__ bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
 
 // Classify the key blocks of one row from its codes: 2 all valid, 1 some valid; with no valid
 // key: 0x82 all 32 keys real (masked), 0x81 some real, 0x80 none.  One wavefront; returns
 // true if the row has a valid key.
-__device__ __forceinline__ bool classify_row(const uint8_t* crow, int nb, int lane, uint8_t* cls) {
+__device__ __forceinline__ bool classify_row(const uint8_t* crow, int nb, int lane, uint8_t* cls,
+                                             unsigned long long& act, unsigned long long& full) {
     bool any_valid = false;
     for (int base = 0; base < nb; base += 64) {
         const int blk = base + lane;
@@ -82,8 +71,10 @@ __device__ __forceinline__ bool classify_row(const uint8_t* crow, int nb, int la
             }
             cls[blk] = nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal == 32 ? 0x82 : (nreal > 0 ? 0x81 : 0x80)));
         }
-        const bool v = __ballot(nvalid > 0) != 0ull;
-        any_valid = any_valid || v;
+        // bit masks of the blocks with a valid key / with only valid keys (first 64 blocks)
+        const unsigned long long va = __ballot(nvalid > 0), vf = __ballot(nvalid == 32);
+        if (base == 0) { act = va; full = vf; }
+        any_valid = any_valid || va != 0ull;
     }
     return any_valid;
 }
@@ -169,6 +160,17 @@ __device__ __forceinline__ float exp_pack_sum(const f32x16& s, bf16x8& p0, bf16x
     return sum16_bf16(a, b);
 }
 
+// Instruction order for a block of NM independent MFMAs and VALU work: one MFMA, then NV VALU
+// instructions, repeated.
+template <int NM, int NV>
+__device__ __forceinline__ void interleave_mfma() {
+    if constexpr (NM > 0) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, NV, 0);
+        interleave_mfma<NM - 1, NV>();
+    }
+}
+
 // A lane's partial row sum above this (or inf / NaN from an overflowed exponent) sends the
 // tile through the exact max-and-rescale path instead.
 constexpr float kSumLimit = 1.0995116e12f;   // 2^40
@@ -210,7 +212,6 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
     __syncthreads();
 
     const bf16x8 kx = slot0_frag(1.0f, half);
-    const bf16x8 id0 = identity_frag(0, col, half), id1 = identity_frag(1, col, half);
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
     // rows are dealt round-robin over the row ranges so that every workgroup gets the same mix
@@ -218,7 +219,8 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
     for (int a = rr + p.rowranges * wave; a < p.nrows; a += p.rowranges * kStripWaves) {
         const size_t row_units = ((size_t)a * H + h) * nb * 128;        // fragment units of (a, h)
         const uint8_t* crow = p.codes + (size_t)a * nb * 32;
-        const bool uni = !classify_row(crow, nb, lane, cls);
+        unsigned long long act = 0, full = 0;
+        const bool uni = !classify_row(crow, nb, lane, cls, act, full);
         bf16x8 q[2][2], qx[2];
         f32x16 o[2][1];
         float m[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
@@ -229,86 +231,136 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
             qx[t] = slot0_frag(0.f, half);
             o[t][0] = zero;
         }
-        bool first = true;
         __builtin_amdgcn_s_waitcnt(0);   // cls bytes written above are read by this wavefront
         __builtin_amdgcn_wave_barrier();
+
+        // scores of query block t against key block kb: bias + (1)(-m) + K Q^T
+        auto score = [&](int t, int kb, const bf16x8& k0, const bf16x8& k1) -> f32x16 {
+            const u32x4* sb = strip + kb * 256 + t * 128 + lane;
+            f32x16 r = bias_tile_acc(sb[0], sb[64]);
+            r = mfma32(kx, qx[t], r);
+            r = mfma32(k0, q[t][0], r);
+            return mfma32(k1, q[t][1], r);
+        };
+        // true maximum of the tile, running maximum moved, partial results rescaled
+        auto renorm = [&](int t, f32x16& st) {
+            rescale<1>(st, tile_max(st), m[t], l[t], o[t], qx[t], half);
+        };
 
         if (uni) {
             // No valid key: every real key gets the same weight (see the masking note on top),
             // whatever the query, so both query blocks get the plain sum of V over real keys.
+            // The V fragments of four blocks are requested before the first is used.
             const bf16x8 ones = as_frag(u32x4{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u});
-            for (int kb = 0; kb < nb; ++kb) {
-                const int c = __builtin_amdgcn_readfirstlane((int)cls[kb]);
-                if (c == 0x80) continue;
-                const u32x4* vp = vf + row_units + kb * 128 + lane;
-                const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
-                bf16x8 p0 = ones, p1 = ones;
-                float cnt = 16.f;
-                if (c != 0x82) {
-                    f32x16 sc = zero;
-                    mask_scores(sc, crow + kb * 32, half, true, 0.f);
-                    cnt = exp_pack_sum(sc, p0, p1);
+            for (int kb0 = 0; kb0 < nb; kb0 += 4) {
+                u32x4 vv[4][2];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const u32x4* vp = vf + row_units + min(kb0 + i, nb - 1) * 128 + lane;
+                    vv[i][0] = vp[0];
+                    vv[i][1] = vp[64];
                 }
-                l[0] += cnt;
-                o[0][0] = mfma32(v0, p0, o[0][0]);
-                o[0][0] = mfma32(v1, p1, o[0][0]);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int kb = kb0 + i;
+                    if (kb >= nb) break;
+                    const int c = __builtin_amdgcn_readfirstlane((int)cls[kb]);
+                    if (c == 0x80) continue;
+                    bf16x8 p0 = ones, p1 = ones;
+                    float cnt = 16.f;
+                    if (c != 0x82) {
+                        f32x16 sc = zero;
+                        mask_scores(sc, crow + kb * 32, half, true, 0.f);
+                        cnt = exp_pack_sum(sc, p0, p1);
+                    }
+                    l[0] += cnt;
+                    o[0][0] = mfma32(as_frag(vv[i][0]), p0, o[0][0]);
+                    o[0][0] = mfma32(as_frag(vv[i][1]), p1, o[0][0]);
+                }
             }
             l[1] = l[0];
             o[1][0] = o[0][0];
-        } else
-        for (int kb = 0; kb < nb; ++kb) {
-            const int c = __builtin_amdgcn_readfirstlane((int)cls[kb]);
-            if (c & 0x80) continue;              // no valid key in this block
-            const u32x4* kp = kf + row_units + kb * 128 + lane;
-            const u32x4* vp = vf + row_units + kb * 128 + lane;
-            const bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
-            const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
-            const u32x4* sb = strip + kb * 256 + lane;
-            f32x16 s[2];
-            auto scores = [&]() {
+        } else {
+            // ---- the first block with a valid key and every block with masked keys: exact
+            // path (mask, true maximum, rescale when it moved by more than 2^8) ------------------
+            const int kfirst = __builtin_ctzll(act);
+            unsigned long long slow = (act & ~full) | (1ull << kfirst);
+            bool first = true;
+            while (slow) {
+                const int kb = __builtin_ctzll(slow);
+                slow &= slow - 1;
+                const bool mixed = !((full >> kb) & 1ull);
+                const u32x4* kp = kf + row_units + kb * 128 + lane;
+                const u32x4* vp = vf + row_units + kb * 128 + lane;
+                const bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
+                const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
 #pragma unroll
                 for (int t = 0; t < 2; ++t) {
-                    s[t] = mfma32(as_frag(sb[t * 128]), id0, zero);
-                    s[t] = mfma32(as_frag(sb[t * 128 + 64]), id1, s[t]);
-                    s[t] = mfma32(kx, qx[t], s[t]);
-                    s[t] = mfma32(k0, q[t][0], s[t]);
-                    s[t] = mfma32(k1, q[t][1], s[t]);
+                    f32x16 st = score(t, kb, k0, k1);
+                    if (mixed) mask_scores(st, crow + kb * 32, half, false, m[t]);
+                    const float mx = tile_max(st);
+                    if (first || __any(mx > kLazyMax)) rescale<1>(st, mx, m[t], l[t], o[t], qx[t], half);
+                    bf16x8 p0, p1;
+                    l[t] += exp_pack_sum(st, p0, p1);
+                    o[t][0] = mfma32(v0, p0, o[t][0]);
+                    o[t][0] = mfma32(v1, p1, o[t][0]);
                 }
-            };
-            // exact path: mask, true maximum, rescale when it moved by more than 2^8
-            auto exact = [&]() {
-                if (c != 2) {
-                    mask_scores(s[0], crow + kb * 32, half, false, m[0]);
-                    mask_scores(s[1], crow + kb * 32, half, false, m[1]);
-                }
-                const float mx0 = tile_max(s[0]), mx1 = tile_max(s[1]);
-                if (first || __any(fmaxf(mx0, mx1) > kLazyMax)) {
-                    rescale<1>(s[0], mx0, m[0], l[0], o[0], qx[0], half);
-                    rescale<1>(s[1], mx1, m[1], l[1], o[1], qx[1], half);
-                }
-            };
-            scores();
-            if (first || c != 2) exact();
-            first = false;
-            // hot path: no maximum at all.  Scores of a row stay within range of its running
-            // maximum unless a later block towers over it; that shows up as a huge row sum.
-            bf16x8 p0[2], p1[2];
-            float ls0 = exp_pack_sum(s[0], p0[0], p1[0]);
-            float ls1 = exp_pack_sum(s[1], p0[1], p1[1]);
-            if (__any(!(fmaxf(ls0, ls1) < kSumLimit))) {
-                scores();
-                first = true;            // force the rescale in exact()
-                exact();
                 first = false;
-                ls0 = exp_pack_sum(s[0], p0[0], p1[0]);
-                ls1 = exp_pack_sum(s[1], p0[1], p1[1]);
             }
-            l[0] += ls0;
-            l[1] += ls1;
-#pragma unroll
-            for (int t = 0; t < 2; ++t) {
-                o[t][0] = mfma32(v0, p0[t], o[t][0]);
-                o[t][0] = mfma32(v1, p1[t], o[t][0]);
+
+            // ---- all other blocks (every key valid): no maximum at all.  Scores of a row stay
+            // within range of its running maximum unless a later block towers over it; that
+            // shows up as a huge row sum and sends the tile through renorm().  The two query
+            // blocks are two independent streams, run half a step apart so that the MFMAs of
+            // one are issued between the exponentials of the other.
+            unsigned long long fm = full & ~(1ull << kfirst);
+            if (fm) {
+                int kb = __builtin_ctzll(fm);
+                fm &= fm - 1;
+                const u32x4* kp = kf + row_units + kb * 128 + lane;
+                const u32x4* vp = vf + row_units + kb * 128 + lane;
+                bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
+                bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
+                f32x16 s0 = score(0, kb, k0, k1), s1;
+                while (true) {
+                    const bool more = fm != 0;
+                    const int kn = more ? __builtin_ctzll(fm) : kb;
+                    fm &= fm - 1;
+                    // -- scores of stream 1 and the next K among the exponentials of stream 0
+                    s1 = score(1, kb, k0, k1);
+                    const u32x4* kpn = kf + row_units + kn * 128 + lane;
+                    const bf16x8 kn0 = as_frag(kpn[0]), kn1 = as_frag(kpn[64]);
+                    bf16x8 p0, p1;
+                    float ls = exp_pack_sum(s0, p0, p1);
+                    interleave_mfma<3, 12>();
+                    if (__any(!(ls < kSumLimit))) {
+                        s0 = score(0, kb, k0, k1);
+                        renorm(0, s0);
+                        ls = exp_pack_sum(s0, p0, p1);
+                    }
+                    l[0] += ls;
+                    // -- PV of stream 0 and its next scores among the exponentials of stream 1
+                    o[0][0] = mfma32(v0, p0, o[0][0]);
+                    o[0][0] = mfma32(v1, p1, o[0][0]);
+                    s0 = score(0, kn, kn0, kn1);
+                    ls = exp_pack_sum(s1, p0, p1);
+                    interleave_mfma<5, 8>();
+                    if (__any(!(ls < kSumLimit))) {
+                        s1 = score(1, kb, k0, k1);
+                        renorm(1, s1);
+                        ls = exp_pack_sum(s1, p0, p1);
+                    }
+                    l[1] += ls;
+                    o[1][0] = mfma32(v0, p0, o[1][0]);
+                    o[1][0] = mfma32(v1, p1, o[1][0]);
+                    if (!more) break;
+                    const u32x4* vpn = vf + row_units + kn * 128 + lane;
+                    v0 = as_frag(vpn[0]);
+                    v1 = as_frag(vpn[64]);
+                    k0 = kn0;
+                    k1 = kn1;
+                    kb = kn;
+                }
             }
         }
 
@@ -377,7 +429,9 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
     };
 
     if (wave < A) {
-        const bool any_valid = classify_row(p.codes + (size_t)rowc(wave) * nb * 32, nb, lane, cls_s[wave]);
+        unsigned long long act_unused, full_unused;
+        const bool any_valid = classify_row(p.codes + (size_t)rowc(wave) * nb * 32, nb, lane, cls_s[wave],
+                                            act_unused, full_unused);
         if (lane == 0) uniform_s[wave] = any_valid ? 0 : 1;
     }
 
@@ -405,7 +459,6 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
     };
 
     const bf16x8 kx = slot0_frag(1.0f, half);
-    const bf16x8 id0 = identity_frag(0, col, half), id1 = identity_frag(1, col, half);
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     bf16x8 q[R][DKS], qx[R];
     f32x16 o[R][DV];
@@ -435,8 +488,8 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
         if (kb + 1 < nb) prefetch(kb + 1);
         const u32x4* st = stage[kb & 1];
         if (wave_active) {
-            const bf16x8 b0 = as_frag(st[BIAS_OFF + qbl * 128 + lane]);
-            const bf16x8 b1 = as_frag(st[BIAS_OFF + qbl * 128 + 64 + lane]);
+            const u32x4 b0 = st[BIAS_OFF + qbl * 128 + lane];
+            const u32x4 b1 = st[BIAS_OFF + qbl * 128 + 64 + lane];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (r >= nr) continue;
@@ -449,8 +502,7 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
                 }
                 f32x16 s;
                 auto scores = [&]() {
-                    s = mfma32(b0, id0, zero);
-                    s = mfma32(b1, id1, s);
+                    s = bias_tile_acc(b0, b1);
                     s = mfma32(kx, qx[r], s);
 #pragma unroll
                     for (int ks = 0; ks < DKS; ++ks)
@@ -581,9 +633,7 @@ int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream) {
         }
         return 0;
     }
-    static const char* env = getenv("KFH_FLASH_STAGED");     // experiment knob
-    if (head_dim_pad == 32 && args.nb <= kStripMaxBlocks && args.nrows >= 4 * kStripWaves &&
-        !(env && env[0] == '1'))
+    if (head_dim_pad == 32 && args.nb <= kStripMaxBlocks && args.nrows >= 4 * kStripWaves)
         return launch_strip(args, stream);
     return launch_staged(args, head_dim_pad, stream);
 }

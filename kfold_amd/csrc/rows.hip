@@ -93,7 +93,7 @@ void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int 
 }
 
 // Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled bf16 tiles (bias_tile_elem layout);
-// one thread writes the 8 queries of one (tile, k-step, lane) slot.
+// one thread writes the 8 keys of one (tile, chunk, lane) slot.
 template <int IO>
 __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __restrict__ tiles,
                                   long long total, int H, int L, int nb) {
@@ -103,14 +103,14 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
     long long t = i >> 7;
     const int kb = (int)(t % nb); t /= nb;
     const int qb = (int)(t % nb); t /= nb;          // t = batch * H + h
-    const int k = kb * 32 + (lane & 31);
+    const int q = qb * 32 + (lane & 31);
     uint32_t w[4];
 #pragma unroll
     for (int e = 0; e < 8; e += 2) {
         float v[2];
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-            const int q = qb * 32 + 16 * c + 8 * (lane >> 5) + e + u;
+            const int k = kb * 32 + acc_row(8 * c + e + u, lane >> 5);
             float x = 0.f;
             if (q < L && k < L) {
                 const size_t off = ((size_t)t * L + q) * L + k;

@@ -90,15 +90,17 @@ def test_pair_bias_projection_and_trunk_apb(n):
                                   ref.linear_pair_bias.weight, device=torch.device(DEV))
         tiles = ops.pair_bias_project(zb.to(DEV), blob, 16)
         nb = (n + 31) // 32
-        # bf16 tiles [h][qb][kb][k-step c][lane = key + 32*half][e]; query = 16c + 8*half + e
+        # bf16 tiles [h][qb][kb][chunk c][lane = query + 32*half][j]: element j of chunk c is
+        # accumulator register v = 8c + j, i.e. key 8*(v//4) + 4*half + v%4
         t1 = tiles.view(torch.bfloat16).view(16, nb, nb, 2, 2, 32, 8).float()
         t2 = tiles_dense.view(torch.bfloat16).view(16, nb, nb, 2, 2, 32, 8).float()
         ar = torch.arange
-        q = (ar(nb)[:, None, None, None] * 32 + 16 * ar(2)[None, :, None, None]
-             + 8 * ar(2)[None, None, :, None] + ar(8)[None, None, None, :])            # [qb, c, half, e]
-        k = ar(nb)[:, None] * 32 + ar(32)[None, :]                                       # [kb, key]
-        valid_q = (q < n)[None, :, None, :, :, None, :]
-        valid_k = (k < n)[None, None, :, None, None, :, None]
+        v = 8 * ar(2)[:, None, None] + ar(8)[None, None, :]                              # [c, 1, j]
+        key32 = 8 * (v // 4) + 4 * ar(2)[None, :, None] + v % 4                          # [c, half, j]
+        k = ar(nb)[:, None, None, None] * 32 + key32[None]                               # [kb, c, half, j]
+        q = ar(nb)[:, None] * 32 + ar(32)[None, :]                                       # [qb, query]
+        valid_q = (q < n)[None, :, None, None, None, :, None]
+        valid_k = (k < n)[None, None, :, :, :, None, :]
         sel = (valid_q & valid_k).expand_as(t1).to(DEV)
         assert_close(t1[sel], t2[sel], "pair bias tiles", max_abs=3e-2, mean_abs=3e-3, rel_fro=1e-2)
 
