@@ -27,6 +27,11 @@ if ROOT not in sys.path:
 
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+CAL_COPY_BYTES = 256 << 20     # size of the counter-calibration copy
+# HBM bytes per launch of the attention kernel at N=768 (FETCH_SIZE + WRITE_SIZE, each scaled by
+# the calibration copy's reading in the same run); the counter runs are summarised in
+# profiles/hot_path_kernels_n768_hbm_traffic.md.  None where no counter run exists.
+MEASURED_TRAFFIC_BYTES = {768: 832469031}
 
 
 def block_flops(n: int) -> dict:
@@ -124,6 +129,15 @@ def main() -> int:
     pm, tok = pm.to(dev), tok.to(dev)
     fl = block_flops(n)
 
+    # One plain device copy of known size (256 MiB read + 256 MiB written).  It plays no part in
+    # the timing; under `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` its counter reading gives the
+    # scale factor of those counters for the `roofline.traffic` figure.
+    cal_src = torch.empty(CAL_COPY_BYTES, dtype=torch.uint8, device=dev)
+    cal_dst = torch.empty_like(cal_src)
+    cal_dst.copy_(cal_src)
+    torch.cuda.synchronize()
+    del cal_src, cal_dst
+
     with torch.inference_mode():
         def step():
             block(z, s, pm, tok, inplace_output=True)
@@ -207,7 +221,7 @@ def main() -> int:
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(n),
             "avg_launch_ms": round(flash_avg, 4),
             "flops_per_launch": flash_flops,
         },
