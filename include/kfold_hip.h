@@ -145,9 +145,11 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
                            int expansion, float eps, int io_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------
- * Pair bias of the token-track attention, as fp32 "bias tiles": the layout the attention
- * kernel reads, [batch][head][query block of 32][key block of 32][4 KiB tile], values
- * pre-multiplied by log2(e).
+ * Pair bias of the token-track attention, as bf16 "bias tiles": the layout the attention
+ * kernel reads, [batch][head][query block of 32][key block of 32][2 KiB tile], values
+ * pre-multiplied by log2(e); inside a tile the 1024 values are in the register order of the
+ * kernel's transposed score accumulator (an opaque layout: produce tiles only with the two
+ * calls below).
  * ------------------------------------------------------------------------------------- */
 size_t kfh_bias_tiles_bytes(int nbatch, int H, int L);
 
