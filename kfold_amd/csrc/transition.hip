@@ -95,29 +95,46 @@ __global__ __launch_bounds__(TILE * 2, 3) void transition_kernel(
         __syncthreads();
     }
 
-    // block n, lane col <-> channel 4*col + n (ROW_INTERLEAVE4)
+    // block n, lane col <-> channel 4*col + n (ROW_INTERLEAVE4).  Rows in two groups of 8: all
+    // residual values of a group are requested before its first store, so one memory latency
+    // is paid per group and, with out aliasing residual, a row is read before it is written.
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const long long p = p0 + wave * 32 + acc_row(v, half);
-        if (p < M) {
-            const size_t e0 = (size_t)p * kC + 4 * col;
-            float o0 = oacc[0][v], o1 = oacc[1][v], o2 = oacc[2][v], o3 = oacc[3][v];
-            const float mk = mask ? (mask[p] ? 1.f : 0.f) : 1.f;
-            if constexpr (IO == KFH_BF16) {
-                if (residual) {
-                    const u32x2 r = *reinterpret_cast<const u32x2*>(
-                        static_cast<const uint16_t*>(residual) + e0);
-                    o0 += bf16_lo(r[0]); o1 += bf16_hi(r[0]); o2 += bf16_lo(r[1]); o3 += bf16_hi(r[1]);
+    for (int g = 0; g < 2; ++g) {
+        u32x2 rb[8];
+        f32x4 rf[8];
+        if (residual) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const long long p = min(p0 + wave * 32 + acc_row(8 * g + u, half), M - 1);
+                const size_t e0 = (size_t)p * kC + 4 * col;
+                if constexpr (IO == KFH_BF16)
+                    rb[u] = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(residual) + e0);
+                else
+                    rf[u] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int v = 8 * g + u;
+            const long long p = p0 + wave * 32 + acc_row(v, half);
+            if (p < M) {
+                const size_t e0 = (size_t)p * kC + 4 * col;
+                float o0 = oacc[0][v], o1 = oacc[1][v], o2 = oacc[2][v], o3 = oacc[3][v];
+                const float mk = mask ? (mask[p] ? 1.f : 0.f) : 1.f;
+                if constexpr (IO == KFH_BF16) {
+                    if (residual) {
+                        o0 += bf16_lo(rb[u][0]); o1 += bf16_hi(rb[u][0]);
+                        o2 += bf16_lo(rb[u][1]); o3 += bf16_hi(rb[u][1]);
+                    }
+                    u32x2 o = {pack_bf16(o0 * mk, o1 * mk), pack_bf16(o2 * mk, o3 * mk)};
+                    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
+                } else {
+                    if (residual) {
+                        o0 += rf[u][0]; o1 += rf[u][1]; o2 += rf[u][2]; o3 += rf[u][3];
+                    }
+                    f32x4 o = {o0 * mk, o1 * mk, o2 * mk, o3 * mk};
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + e0) = o;
                 }
-                u32x2 o = {pack_bf16(o0 * mk, o1 * mk), pack_bf16(o2 * mk, o3 * mk)};
-                *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
-            } else {
-                if (residual) {
-                    const f32x4 r = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
-                    o0 += r[0]; o1 += r[1]; o2 += r[2]; o3 += r[3];
-                }
-                f32x4 o = {o0 * mk, o1 * mk, o2 * mk, o3 * mk};
-                *reinterpret_cast<f32x4*>(static_cast<float*>(out) + e0) = o;
             }
         }
     }

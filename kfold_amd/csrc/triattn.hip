@@ -26,7 +26,7 @@
 namespace kfh {
 
 constexpr int kH = 4;          // heads
-constexpr int kTileA = 256;    // positions per workgroup in proj/out kernels (64 per wavefront)
+constexpr int kTileA = 256;    // positions per workgroup in proj/out kernels (32 per wavefront)
 
 __device__ __forceinline__ size_t frag_index(int a, int h, int blk, int ks, int nb, int lane) {
     return ((((size_t)a * kH + h) * nb + blk) * 2 + ks) * 64 + lane;
@@ -186,66 +186,75 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
 }
 
 // ------------------------------------------------------------------------------------------
-// output projection: out'[a][b] = W_o (gated o), 64 positions per wavefront
+// output projection: out'[a][b] = W_o (gated o), 32 positions per wavefront, 8 wavefronts
 // ------------------------------------------------------------------------------------------
 template <int IO>
-__global__ __launch_bounds__(256) void triattn_out_kernel(
+__global__ __launch_bounds__(512, 3) void triattn_out_kernel(
     const bf16x8* __restrict__ of, const char* __restrict__ blob, const void* residual, void* out,
     int N, int nb, int ending) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
     const int a = blockIdx.y, t0 = blockIdx.x * kTileA;
-    const int blk0 = (t0 + wave * 64) >> 5;
-    if (blk0 >= nb) return;
-    const bool two = blk0 + 1 < nb;
+    const int blk = (t0 >> 5) + wave;
+    if (blk >= nb) return;
 
-    bf16x8 xf[2][kKS];
+    bf16x8 xf[kKS];
 #pragma unroll
-    for (int pb = 0; pb < 2; ++pb) {
-        const int blk = (pb == 0 || two) ? blk0 + pb : blk0;
-#pragma unroll
-        for (int h = 0; h < kH; ++h) {
-            xf[pb][2 * h] = of[frag_index(a, h, blk, 0, nb, lane)];
-            xf[pb][2 * h + 1] = of[frag_index(a, h, blk, 1, nb, lane)];
-        }
+    for (int h = 0; h < kH; ++h) {
+        xf[2 * h] = of[frag_index(a, h, blk, 0, nb, lane)];
+        xf[2 * h + 1] = of[frag_index(a, h, blk, 1, nb, lane)];
     }
-    f32x16 acc[2][4];
-#pragma unroll
-    for (int pb = 0; pb < 2; ++pb)
-#pragma unroll
-        for (int n = 0; n < 4; ++n)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[pb][n][v] = 0.f;
-    const bf16x8* wo = reinterpret_cast<const bf16x8*>(blob + kTaOutOff);
+    auto elem0 = [&](int v) -> size_t {
+        const int b = min(blk * 32 + acc_row(v, half), N - 1);
+        const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
+        return pos * kC + 4 * col;
+    };
+
+    f32x16 acc[4];
 #pragma unroll
     for (int n = 0; n < 4; ++n)
 #pragma unroll
-        for (int ks = 0; ks < kKS; ++ks) {
-            const bf16x8 w = wo[(n * kKS + ks) * 64 + lane];
-            acc[0][n] = mfma32(xf[0][ks], w, acc[0][n]);
-            acc[1][n] = mfma32(xf[1][ks], w, acc[1][n]);
+        for (int v = 0; v < 16; ++v) acc[n][v] = 0.f;
+    const bf16x8* wo = reinterpret_cast<const bf16x8*>(blob + kTaOutOff);
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks) acc[n] = mfma32(xf[ks], wo[(n * kKS + ks) * 64 + lane], acc[n]);
+        __builtin_amdgcn_sched_barrier(0);      // keep the weight loads of later blocks out of flight
+    }
+    // Rows in two groups of 8: all residual values of a group are requested before its first
+    // store, so one memory latency is paid per group and, with out aliasing residual, a row is
+    // read before it is written.
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+        u32x2 rb[8];
+        f32x4 rf[8];
+        if (residual) {
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if constexpr (IO == KFH_BF16)
+                    rb[u] = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(residual) + elem0(8 * g + u));
+                else
+                    rf[u] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + elem0(8 * g + u));
+            }
         }
 #pragma unroll
-    for (int pb = 0; pb < 2; ++pb) {
-        if (pb == 1 && !two) break;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int b = (blk0 + pb) * 32 + acc_row(v, half);
+        for (int u = 0; u < 8; ++u) {
+            const int v = 8 * g + u;
+            const int b = blk * 32 + acc_row(v, half);
             if (b < N) {
-                const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
-                const size_t e0 = pos * kC + 4 * col;
-                float o0 = acc[pb][0][v], o1 = acc[pb][1][v], o2 = acc[pb][2][v], o3 = acc[pb][3][v];
+                const size_t e0 = elem0(v);
+                float o0 = acc[0][v], o1 = acc[1][v], o2 = acc[2][v], o3 = acc[3][v];
                 if constexpr (IO == KFH_BF16) {
                     if (residual) {
-                        const u32x2 r = *reinterpret_cast<const u32x2*>(
-                            static_cast<const uint16_t*>(residual) + e0);
+                        const u32x2 r = rb[u];
                         o0 += bf16_lo(r[0]); o1 += bf16_hi(r[0]); o2 += bf16_lo(r[1]); o3 += bf16_hi(r[1]);
                     }
                     u32x2 o = {pack_bf16(o0, o1), pack_bf16(o2, o3)};
                     *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
                 } else {
                     if (residual) {
-                        const f32x4 r = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
+                        const f32x4 r = rf[u];
                         o0 += r[0]; o1 += r[1]; o2 += r[2]; o3 += r[3];
                     }
                     f32x4 o = {o0, o1, o2, o3};
@@ -284,10 +293,10 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
     if (!(stages & KFH_STAGE_OUT)) return;
 
     if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, block, 0, stream, of, blob,
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, dim3(512), 0, stream, of, blob,
                            residual, out, N, nb, ending);
     else
-        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, block, 0, stream, of, blob,
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, dim3(512), 0, stream, of, blob,
                            residual, out, N, nb, ending);
 }
 

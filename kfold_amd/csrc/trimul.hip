@@ -170,7 +170,7 @@ void launch_trimul_in(const void* z, int io_dtype, const uint8_t* mask, const ch
 // output phase: 128 positions of one row i per workgroup, 32 per wavefront
 // -----------------------------------------------------------------------------------------
 template <int IO>
-__global__ __launch_bounds__(256) void trimul_out_kernel(
+__global__ __launch_bounds__(256, 4) void trimul_out_kernel(
     const uint16_t* __restrict__ planes_y, const uint16_t* __restrict__ gate,
     const char* __restrict__ blob, const void* residual, void* out, int N, int Np, float eps) {
     __shared__ __attribute__((aligned(16))) char yt[kC * kXS];   // [d][128 positions] bf16
@@ -227,37 +227,58 @@ __global__ __launch_bounds__(256) void trimul_out_kernel(
         for (int v = 0; v < 16; ++v) acc[nb][v] = 0.f;
     const bf16x8* wo = reinterpret_cast<const bf16x8*>(blob + kTmOutOff);
 #pragma unroll
-    for (int nb = 0; nb < 4; ++nb)
+    for (int nb = 0; nb < 4; ++nb) {
 #pragma unroll
         for (int ks = 0; ks < kKS; ++ks)
             acc[nb] = mfma32(yf[ks], wo[(nb * kKS + ks) * 64 + lane], acc[nb]);
+        __builtin_amdgcn_sched_barrier(0);      // keep the weight loads of later blocks out of flight
+    }
 
-    // block nb, lane col <-> channel 4*col + nb (ROW_INTERLEAVE4): 8 or 16 contiguous bytes per lane
+    // block nb, lane col <-> channel 4*col + nb (ROW_INTERLEAVE4): 8 or 16 contiguous bytes per
+    // lane.  Rows in two groups of 8: all gate and residual values of a group are requested
+    // before its first store, so one memory latency is paid per group and, with out aliasing
+    // residual, a row is read before it is written.
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int j = j0 + 32 * wave + acc_row(v, half);
-        if (j < N) {
-            const size_t e0 = ((size_t)i * N + j) * kC + 4 * col;
-            const u32x2 g = *reinterpret_cast<const u32x2*>(gate + e0);
-            float o0 = acc[0][v] * bf16_lo(g[0]);
-            float o1 = acc[1][v] * bf16_hi(g[0]);
-            float o2 = acc[2][v] * bf16_lo(g[1]);
-            float o3 = acc[3][v] * bf16_hi(g[1]);
-            if constexpr (IO == KFH_BF16) {
-                if (residual) {
-                    const u32x2 r = *reinterpret_cast<const u32x2*>(
-                        static_cast<const uint16_t*>(residual) + e0);
-                    o0 += bf16_lo(r[0]); o1 += bf16_hi(r[0]); o2 += bf16_lo(r[1]); o3 += bf16_hi(r[1]);
+    for (int g = 0; g < 2; ++g) {
+        u32x2 gv[8];
+        u32x2 rb[8];
+        f32x4 rf[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int j = j0 + 32 * wave + acc_row(8 * g + u, half);
+            const size_t e0 = ((size_t)i * N + min(j, N - 1)) * kC + 4 * col;
+            gv[u] = *reinterpret_cast<const u32x2*>(gate + e0);
+            if (residual) {
+                if constexpr (IO == KFH_BF16)
+                    rb[u] = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(residual) + e0);
+                else
+                    rf[u] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int v = 8 * g + u;
+            const int j = j0 + 32 * wave + acc_row(v, half);
+            if (j < N) {
+                const size_t e0 = ((size_t)i * N + j) * kC + 4 * col;
+                float o0 = acc[0][v] * bf16_lo(gv[u][0]);
+                float o1 = acc[1][v] * bf16_hi(gv[u][0]);
+                float o2 = acc[2][v] * bf16_lo(gv[u][1]);
+                float o3 = acc[3][v] * bf16_hi(gv[u][1]);
+                if constexpr (IO == KFH_BF16) {
+                    if (residual) {
+                        o0 += bf16_lo(rb[u][0]); o1 += bf16_hi(rb[u][0]);
+                        o2 += bf16_lo(rb[u][1]); o3 += bf16_hi(rb[u][1]);
+                    }
+                    u32x2 o = {pack_bf16(o0, o1), pack_bf16(o2, o3)};
+                    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
+                } else {
+                    if (residual) {
+                        o0 += rf[u][0]; o1 += rf[u][1]; o2 += rf[u][2]; o3 += rf[u][3];
+                    }
+                    f32x4 o = {o0, o1, o2, o3};
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + e0) = o;
                 }
-                u32x2 o = {pack_bf16(o0, o1), pack_bf16(o2, o3)};
-                *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + e0) = o;
-            } else {
-                if (residual) {
-                    const f32x4 r = *reinterpret_cast<const f32x4*>(static_cast<const float*>(residual) + e0);
-                    o0 += r[0]; o1 += r[1]; o2 += r[2]; o3 += r[3];
-                }
-                f32x4 o = {o0, o1, o2, o3};
-                *reinterpret_cast<f32x4*>(static_cast<float*>(out) + e0) = o;
             }
         }
     }
