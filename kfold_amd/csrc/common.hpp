@@ -177,18 +177,25 @@ __device__ __forceinline__ void stage_ln_rows(char* tile, const void* src, const
     float gam[8], bet[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) { gam[i] = lnp[ch * 8 + i]; bet[i] = lnp[kC + ch * 8 + i]; }
-#pragma unroll 2
-    for (int it = 0; it < ROWS / RG; ++it) {
-        const int row = it * RG + r16;
-        const long long off = row_off(row);
-        float x[8];
-        if (off >= 0) {
-            load8<IO>(src, (size_t)off + ch * 8, x);
-        } else {
+    // all rows of this thread are requested before the first is normalised: one memory latency
+    // per tile instead of one per row
+    constexpr int NIT = ROWS / RG;
+    float x[NIT][8];
+    bool valid[NIT];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) x[i] = 0.f;
+    for (int it = 0; it < NIT; ++it) {
+        const long long off = row_off(it * RG + r16);
+        valid[it] = off >= 0;
+        load8<IO>(src, (size_t)(valid[it] ? off : 0) + ch * 8, x[it]);
+    }
+#pragma unroll
+    for (int it = 0; it < NIT; ++it) {
+        const int row = it * RG + r16;
+        if (!valid[it]) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) x[it][i] = 0.f;
         }
-        *reinterpret_cast<u32x4*>(tile + row * kXS + ch * 16) = ln_row16(x, gam, bet, eps);
+        *reinterpret_cast<u32x4*>(tile + row * kXS + ch * 16) = ln_row16(x[it], gam, bet, eps);
     }
 }
 

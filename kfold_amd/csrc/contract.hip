@@ -13,7 +13,6 @@
 // ids are dealt round-robin over the 8 XCDs): the two planes of a channel are then read
 // from HBM once and served from that XCD's L2 afterwards.
 #include "kernels.hpp"
-#include <cstdlib>
 
 namespace kfh {
 
@@ -189,20 +188,13 @@ __global__ __launch_bounds__(256, OCC) void contract_kernel(const uint16_t* __re
 
 void launch_contract(const uint16_t* planes_a, const uint16_t* planes_b, uint16_t* planes_y,
                      int Np, int D, hipStream_t stream) {
-    // Np is a multiple of 128; use 256x256 tiles when they divide it, else 128x128
-    static const int variant = getenv("KFH_CONTRACT") ? atoi(getenv("KFH_CONTRACT")) : 0;
-    if (Np % 256 == 0 && variant == 0) {
+    // Np is a multiple of 128; use 256x256 tiles when they divide it, else 128x128.
+    // (192x256 tiles fill the CUs evenly at Np = 768, 6 rounds instead of 4.5, but measured
+    // slower: 189 against 161-177 us.)
+    if (Np % 256 == 0) {
         const int t = Np / 256;
         hipLaunchKernelGGL((contract_kernel<4, 4, 64, 1>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
                            planes_b, planes_y, Np, t, t);
-    } else if (Np % 256 == 0 && variant == 1) {
-        const int tm = Np / 256, tn = Np / 128;
-        hipLaunchKernelGGL((contract_kernel<4, 2, 32, 2>), dim3(D * tm * tn), dim3(256), 0, stream, planes_a,
-                           planes_b, planes_y, Np, tm, tn);
-    } else if (Np % 256 == 0 && variant == 2) {
-        const int tm = Np / 128, tn = Np / 256;
-        hipLaunchKernelGGL((contract_kernel<2, 4, 32, 2>), dim3(D * tm * tn), dim3(256), 0, stream, planes_a,
-                           planes_b, planes_y, Np, tm, tn);
     } else {
         const int t = Np / 128;
         hipLaunchKernelGGL((contract_kernel<2, 2, 64, 2>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
