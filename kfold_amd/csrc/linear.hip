@@ -45,8 +45,36 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
     for (int v = 0; v < 16; ++v) { acc[v] = 0.f; acc2[v] = 0.f; }
     constexpr bool W_IS_A = (EPI == EPI_FRAG_CH);
     constexpr bool TWO = (EPI == EPI_SWIGLU || EPI == EPI_ADALN);
-#pragma unroll 4
-    for (int ks = 0; ks < ksteps; ++ks) {
+    // K is walked in chunks of 8 k-steps; the operands of chunk c+1 are
+    // requested before the MFMAs of chunk c, so one memory latency is paid per 8 k-steps at most
+    constexpr int CH = 8;
+    bf16x8 xa[CH], wa[CH], va[CH], xb[CH], wb2[CH], vb[CH];
+    auto load = [&](int c, bf16x8 (&x)[CH], bf16x8 (&w)[CH], bf16x8 (&v)[CH]) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            x[i] = afrag(c * CH + i);
+            w[i] = W[(size_t)(c * CH + i) * 64];
+            if constexpr (TWO) v[i] = W2[(size_t)(c * CH + i) * 64];
+        }
+    };
+    auto compute = [&](const bf16x8 (&x)[CH], const bf16x8 (&w)[CH], const bf16x8 (&v)[CH]) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            acc = W_IS_A ? mfma32(w[i], x[i], acc) : mfma32(x[i], w[i], acc);
+            if constexpr (TWO) acc2 = mfma32(x[i], v[i], acc2);
+        }
+    };
+    const int nch = ksteps / CH;
+    if (nch > 0) load(0, xa, wa, va);
+    for (int c = 0; c < nch; c += 2) {
+        if (c + 1 < nch) load(c + 1, xb, wb2, vb);
+        compute(xa, wa, va);
+        if (c + 1 < nch) {
+            if (c + 2 < nch) load(c + 2, xa, wa, va);
+            compute(xb, wb2, vb);
+        }
+    }
+    for (int ks = nch * CH; ks < ksteps; ++ks) {      // K not a multiple of 128
         const bf16x8 x = afrag(ks);
         const bf16x8 w = W[(size_t)ks * 64];
         acc = W_IS_A ? mfma32(w, x, acc) : mfma32(x, w, acc);
