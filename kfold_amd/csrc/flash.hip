@@ -55,21 +55,26 @@ __device__ __forceinline__ bf16x8 as_frag(u32x4 v) { return __builtin_bit_cast(b
 // Classify the key blocks of one row from its codes: 2 all valid, 1 some valid; with no valid
 // key: 0x82 all 32 keys real (masked), 0x81 some real, 0x80 none.  One wavefront; returns
 // true if the row has a valid key.
+__device__ __forceinline__ int classify_block(const u32x4& c0, const u32x4& c1, int& nvalid) {
+    int nreal = 0;
+    nvalid = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        nvalid += __popc(c0[i] & 0x02020202u) + __popc(c1[i] & 0x02020202u);
+        nreal += __popc(c0[i] & 0x03030303u) + __popc(c1[i] & 0x03030303u);
+    }
+    return nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal == 32 ? 0x82 : (nreal > 0 ? 0x81 : 0x80)));
+}
+
 __device__ __forceinline__ bool classify_row(const uint8_t* crow, int nb, int lane, uint8_t* cls,
                                              unsigned long long& act, unsigned long long& full) {
     bool any_valid = false;
     for (int base = 0; base < nb; base += 64) {
         const int blk = base + lane;
-        int nvalid = 0, nreal = 0;
+        int nvalid = 0;
         if (blk < nb) {
             const u32x4* c = reinterpret_cast<const u32x4*>(crow + blk * 32);
-            const u32x4 c0 = c[0], c1 = c[1];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                nvalid += __popc(c0[i] & 0x02020202u) + __popc(c1[i] & 0x02020202u);
-                nreal += __popc(c0[i] & 0x03030303u) + __popc(c1[i] & 0x03030303u);
-            }
-            cls[blk] = nvalid == 32 ? 2 : (nvalid > 0 ? 1 : (nreal == 32 ? 0x82 : (nreal > 0 ? 0x81 : 0x80)));
+            cls[blk] = classify_block(c[0], c[1], nvalid);
         }
         // bit masks of the blocks with a valid key / with only valid keys (first 64 blocks)
         const unsigned long long va = __ballot(nvalid > 0), vf = __ballot(nvalid == 32);
@@ -216,18 +221,37 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
 
     // rows are dealt round-robin over the row ranges so that every workgroup gets the same mix
     // of padded and valid rows
-    for (int a = rr + p.rowranges * wave; a < p.nrows; a += p.rowranges * kStripWaves) {
+    // The q fragments and key codes of a row are requested while the previous row of this
+    // wavefront is being finished.
+    u32x4 nq[4], nc[2];
+    auto request_row = [&](int a) {
+        const size_t ru = ((size_t)a * H + h) * nb * 128;
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            nq[2 * t] = qf[ru + qb[t] * 128 + lane];
+            nq[2 * t + 1] = qf[ru + qb[t] * 128 + 64 + lane];
+        }
+        const u32x4* c = reinterpret_cast<const u32x4*>(p.codes + (size_t)a * nb * 32 + min(lane, nb - 1) * 32);
+        nc[0] = c[0];
+        nc[1] = c[1];
+    };
+    const int a_first = rr + p.rowranges * wave, a_step = p.rowranges * kStripWaves;
+    if (a_first < p.nrows) request_row(a_first);
+    for (int a = a_first; a < p.nrows; a += a_step) {
         const size_t row_units = ((size_t)a * H + h) * nb * 128;        // fragment units of (a, h)
         const uint8_t* crow = p.codes + (size_t)a * nb * 32;
-        unsigned long long act = 0, full = 0;
-        const bool uni = !classify_row(crow, nb, lane, cls, act, full);
+        int nvalid = 0;
+        const int c_lane = classify_block(nc[0], nc[1], nvalid);
+        if (lane < nb) cls[lane] = (uint8_t)c_lane; else nvalid = 0;
+        const unsigned long long act = __ballot(nvalid > 0), full = __ballot(nvalid == 32);
+        const bool uni = act == 0ull;
         bf16x8 q[2][2], qx[2];
         f32x16 o[2][1];
         float m[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            q[t][0] = as_frag(qf[row_units + qb[t] * 128 + lane]);
-            q[t][1] = as_frag(qf[row_units + qb[t] * 128 + 64 + lane]);
+            q[t][0] = as_frag(nq[2 * t]);
+            q[t][1] = as_frag(nq[2 * t + 1]);
             qx[t] = slot0_frag(0.f, half);
             o[t][0] = zero;
         }
@@ -364,12 +388,19 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
             }
         }
 
+        u32x4 gg[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            gg[t][0] = gf[row_units + qb[t] * 128 + lane];
+            gg[t][1] = gf[row_units + qb[t] * 128 + 64 + lane];
+        }
+        if (a + a_step < p.nrows) request_row(a + a_step);
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             if (t == 1 && !have_b) break;
             const float inv = fast_rcp(xhalf_sum(l[t]));
             const size_t u0 = row_units + qb[t] * 128 + lane;
-            const u32x4 g0 = gf[u0], g1 = gf[u0 + 64];
+            const u32x4 g0 = gg[t][0], g1 = gg[t][1];
             f32x16 og;
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
