@@ -98,3 +98,22 @@ def test_triattn_ending_is_transposed_starting_batch_residual_determinism():
         xin = xd.clone()
         ops.triattn_forward(xin, md, blob, 4, True, residual=xin, out=xin)
         assert_close(xin, x.float() + want, "triattn residual in place", rel_fro=5e-3)
+
+
+def test_triattn_long_sequence_sampled_rows():
+    """N = 1248 (39 key blocks: beyond the LDS strip of the short-sequence attention kernel, so
+    the staged kernel runs).  The oracle is evaluated on a sample of rows only: rows are
+    independent given the pair bias, which is computed for the whole tensor."""
+    print("case triattn n=1248 sampled rows", flush=True)
+    n, n_pad = 1248, 40
+    ref, hip = _modules(True, seed=5)
+    x, _, pm = synthetic.pair_inputs(n, 128, n_pad, seed=21)
+    xb = x.to(torch.bfloat16)
+    rows = [0, 1, 617, 1207, 1208, 1247]          # valid rows, the last valid row, padded rows
+    with torch.no_grad():
+        got = hip(xb.to(DEV), pm.to(DEV))[0, rows].float().cpu()
+        xn = ref.layer_norm(xb.float())
+        bias = ref.linear(xn).movedim(-1, -3).unsqueeze(-4)
+        mask5 = pm.float()[..., :, None, None, :]
+        want = ref.mha(xn[:, rows], xn[:, rows], bias, mask5[:, rows])[0]
+    assert_close(got, want, "triattn n=1248 sampled rows")
