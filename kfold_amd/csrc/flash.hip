@@ -112,10 +112,13 @@ __device__ __forceinline__ float tile_max(const f32x16& s) {
 // move the running maximum by (bf16-rounded) mx and rescale the partial results
 template <int DV>
 __device__ __forceinline__ void rescale(f32x16& s, float mx, float& m, float& l, f32x16 (&o)[DV],
-                                        bf16x8& qx, int half) {
-    const float m_new = bf16_lo(pack_bf16(m + mx, 0.f));
+                                        bf16x8& qx, int half, bool fresh) {
+    // `fresh`: nothing accumulated yet (m = 0, l = 0, o = 0): the maximum may start anywhere,
+    // and nothing needs scaling.  Afterwards the maximum only rises, so alpha <= 1 (a large
+    // downward move would scale by exp2(+big) = inf).
+    const float m_new = bf16_lo(pack_bf16(fresh ? mx : m + fmaxf(mx, 0.f), 0.f));
     const float delta = m_new - m;
-    const float alpha = fast_exp2(-delta);
+    const float alpha = fresh ? 1.0f : fast_exp2(-delta);
     m = m_new;
     qx = slot0_frag(-m_new, half);
     l *= alpha;
@@ -151,18 +154,25 @@ __device__ __forceinline__ float sum16_bf16(const u32x4& a, const u32x4& b) {
 }
 
 // p = bf16(exp2(s)) as the two B-operand fragments of the PV product; returns this lane's
-// partial row sum of the *rounded* probabilities, so the normaliser matches what the MFMA
-// accumulates.
+// partial row sum, taken over the fp32 exponentials with plain adds.  (A v_dot2c chain over the
+// rounded bf16 values needs half the instructions, but DOT instructions do not overlap with
+// MFMAs of other wavefronts: measured, 14 MFMAs + 32 v_dot2c take the sum of their times.  The
+// rounding of p is unbiased, so numerator and normaliser still agree to well below bf16.)
 __device__ __forceinline__ float exp_pack_sum(const f32x16& s, bf16x8& p0, bf16x8& p1) {
+    f32x16 e;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) e[v] = fast_exp2(s[v]);
     u32x4 a, b;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        a[i] = pack_bf16(fast_exp2(s[2 * i]), fast_exp2(s[2 * i + 1]));
-        b[i] = pack_bf16(fast_exp2(s[8 + 2 * i]), fast_exp2(s[8 + 2 * i + 1]));
+        a[i] = pack_bf16(e[2 * i], e[2 * i + 1]);
+        b[i] = pack_bf16(e[8 + 2 * i], e[8 + 2 * i + 1]);
     }
     p0 = __builtin_bit_cast(bf16x8, a);
     p1 = __builtin_bit_cast(bf16x8, b);
-    return sum16_bf16(a, b);
+    const float t0 = (e[0] + e[1]) + (e[2] + e[3]), t1 = (e[4] + e[5]) + (e[6] + e[7]);
+    const float t2 = (e[8] + e[9]) + (e[10] + e[11]), t3 = (e[12] + e[13]) + (e[14] + e[15]);
+    return (t0 + t1) + (t2 + t3);
 }
 
 // Instruction order for a block of NM independent MFMAs and VALU work: one MFMA, then NV VALU
@@ -268,7 +278,7 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
         };
         // true maximum of the tile, running maximum moved, partial results rescaled
         auto renorm = [&](int t, f32x16& st) {
-            rescale<1>(st, tile_max(st), m[t], l[t], o[t], qx[t], half);
+            rescale<1>(st, tile_max(st), m[t], l[t], o[t], qx[t], half, false);
         };
 
         if (uni) {
@@ -305,39 +315,13 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
             l[1] = l[0];
             o[1][0] = o[0][0];
         } else {
-            // ---- the first block with a valid key and every block with masked keys: exact
-            // path (mask, true maximum, rescale when it moved by more than 2^8) ------------------
-            const int kfirst = __builtin_ctzll(act);
-            unsigned long long slow = (act & ~full) | (1ull << kfirst);
-            bool first = true;
-            while (slow) {
-                const int kb = __builtin_ctzll(slow);
-                slow &= slow - 1;
-                const bool mixed = !((full >> kb) & 1ull);
-                const u32x4* kp = kf + row_units + kb * 128 + lane;
-                const u32x4* vp = vf + row_units + kb * 128 + lane;
-                const bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
-                const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
-#pragma unroll
-                for (int t = 0; t < 2; ++t) {
-                    f32x16 st = score(t, kb, k0, k1);
-                    if (mixed) mask_scores(st, crow + kb * 32, half, false, m[t]);
-                    const float mx = tile_max(st);
-                    if (first || __any(mx > kLazyMax)) rescale<1>(st, mx, m[t], l[t], o[t], qx[t], half);
-                    bf16x8 p0, p1;
-                    l[t] += exp_pack_sum(st, p0, p1);
-                    o[t][0] = mfma32(v0, p0, o[t][0]);
-                    o[t][0] = mfma32(v1, p1, o[t][0]);
-                }
-                first = false;
-            }
-
-            // ---- all other blocks (every key valid): no maximum at all.  Scores of a row stay
-            // within range of its running maximum unless a later block towers over it; that
-            // shows up as a huge row sum and sends the tile through renorm().  The two query
-            // blocks are two independent streams, run half a step apart so that the MFMAs of
-            // one are issued between the exponentials of the other.
-            unsigned long long fm = full & ~(1ull << kfirst);
+            // ---- Max-free pass over every block with a valid key.  The running maximum starts
+            // at 0 (exp2 domain: logits are a few units wide in practice) and only moves when a
+            // lane's partial row sum exceeds 2^40: then the tile is recomputed through the true
+            // maximum (renorm).  First the blocks whose keys are all valid: the two query blocks
+            // are two independent streams, run half a step apart so that the MFMAs of one are
+            // issued between the exponentials of the other.
+            unsigned long long fm = full;
             if (fm) {
                 int kb = __builtin_ctzll(fm);
                 fm &= fm - 1;
@@ -384,6 +368,68 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
                     k0 = kn0;
                     k1 = kn1;
                     kb = kn;
+                }
+            }
+            // blocks with masked keys, same max-free rule, one block at a time
+            unsigned long long mixed = act & ~full;
+            while (mixed) {
+                const int kb = __builtin_ctzll(mixed);
+                mixed &= mixed - 1;
+                const u32x4* kp = kf + row_units + kb * 128 + lane;
+                const u32x4* vp = vf + row_units + kb * 128 + lane;
+                const bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
+                const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    f32x16 st = score(t, kb, k0, k1);
+                    mask_scores(st, crow + kb * 32, half, false, 0.f);
+                    bf16x8 p0, p1;
+                    float ls = exp_pack_sum(st, p0, p1);
+                    if (__any(!(ls < kSumLimit))) {
+                        st = score(t, kb, k0, k1);
+                        mask_scores(st, crow + kb * 32, half, false, 0.f);
+                        renorm(t, st);
+                        ls = exp_pack_sum(st, p0, p1);
+                    }
+                    l[t] += ls;
+                    o[t][0] = mfma32(v0, p0, o[t][0]);
+                    o[t][0] = mfma32(v1, p1, o[t][0]);
+                }
+            }
+            // ---- Every exponential underflowed (all logits of a query below -100 or so) or
+            // something overflowed to NaN: redo the row with the true running maximum, block by
+            // block (mask, maximum, rescale when it moved by more than 2^8).
+            const float lt0 = xhalf_sum(l[0]), lt1 = xhalf_sum(l[1]);
+            if (__any(!(fminf(lt0, lt1) > 1e-30f))) {
+#pragma unroll
+                for (int t = 0; t < 2; ++t) {
+                    qx[t] = slot0_frag(0.f, half);
+                    o[t][0] = zero;
+                    m[t] = 0.f;
+                    l[t] = 0.f;
+                }
+                unsigned long long todo = act;
+                bool first = true;
+                while (todo) {
+                    const int kb = __builtin_ctzll(todo);
+                    todo &= todo - 1;
+                    const bool mixed = !((full >> kb) & 1ull);
+                    const u32x4* kp = kf + row_units + kb * 128 + lane;
+                    const u32x4* vp = vf + row_units + kb * 128 + lane;
+                    const bf16x8 k0 = as_frag(kp[0]), k1 = as_frag(kp[64]);
+                    const bf16x8 v0 = as_frag(vp[0]), v1 = as_frag(vp[64]);
+#pragma unroll
+                    for (int t = 0; t < 2; ++t) {
+                        f32x16 st = score(t, kb, k0, k1);
+                        if (mixed) mask_scores(st, crow + kb * 32, half, false, m[t]);
+                        const float mx = tile_max(st);
+                        if (first || __any(mx > kLazyMax)) rescale<1>(st, mx, m[t], l[t], o[t], qx[t], half, first);
+                        bf16x8 p0, p1;
+                        l[t] += exp_pack_sum(st, p0, p1);
+                        o[t][0] = mfma32(v0, p0, o[t][0]);
+                        o[t][0] = mfma32(v1, p1, o[t][0]);
+                    }
+                    first = false;
                 }
             }
         }
@@ -539,20 +585,20 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
                     for (int ks = 0; ks < DKS; ++ks)
                         s = mfma32(as_frag(st[(ra * DKS + ks) * 64 + lane]), q[r][ks], s);
                 };
-                auto exact = [&](bool force) {
+                auto exact = [&](bool force, bool fresh) {
                     if (cls != 2)
                         mask_scores(s, p.codes + (size_t)(a0 + ra) * nb * 32 + kb * 32, half, uni, m[r]);
                     const float mx = tile_max(s);
-                    if (force || __any(mx > kLazyMax)) rescale<DV>(s, mx, m[r], l[r], o[r], qx[r], half);
+                    if (force || __any(mx > kLazyMax)) rescale<DV>(s, mx, m[r], l[r], o[r], qx[r], half, fresh);
                 };
                 scores();
-                if (first[r] || cls != 2) exact(first[r]);
+                if (first[r] || cls != 2) exact(first[r], first[r]);
                 first[r] = false;
                 bf16x8 p0, p1;
                 float ls = exp_pack_sum(s, p0, p1);
                 if (__any(!(ls < kSumLimit))) {      // a block towering over the running maximum
                     scores();
-                    exact(true);
+                    exact(true, false);
                     ls = exp_pack_sum(s, p0, p1);
                 }
                 l[r] += ls;

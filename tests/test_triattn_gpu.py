@@ -117,3 +117,23 @@ def test_triattn_long_sequence_sampled_rows():
         mask5 = pm.float()[..., :, None, None, :]
         want = ref.mha(xn[:, rows], xn[:, rows], bias, mask5[:, rows])[0]
     assert_close(got, want, "triattn n=1248 sampled rows")
+
+
+@pytest.mark.parametrize("shift", [-256.0, 256.0, 60.0])
+def test_triattn_logits_far_from_zero(shift):
+    """A pair bias that is a large constant for every (query, key): the softmax is invariant to it,
+    but exp2 of the raw logits under- or overflows, so the kernel has to fall back to the exact
+    running-maximum path (negative shift) or move the maximum on the first block (positive)."""
+    print(f"case triattn bias shift {shift}", flush=True)
+    ref, hip = _modules(True, seed=9, std=0.05)
+    with torch.no_grad():
+        # LN(x) sums to 128 over the channels (gamma = 1, beta = 1), so a constant weight gives
+        # bias = shift for every head, query and key: exactly representable in the bf16 bias
+        # tiles, while q.k still varies
+        ref.layer_norm.bias.fill_(1.0)
+        ref.linear.weight.fill_(shift / 128.0)
+    hip.load_state_dict(ref.state_dict())
+    n = 96
+    x, _, pm = synthetic.pair_inputs(n, 128, 9, seed=13)
+    got, want = _run(ref, hip, x, pm, torch.bfloat16)
+    assert_close(got, want, f"triattn bias shift {shift}", auto_scale=True)
