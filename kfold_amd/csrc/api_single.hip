@@ -311,12 +311,14 @@ int kfh_transition_pack(const void* ln_w, const void* ln_b, const void* swiglu_w
         const int nstep = hid / 32;
         for (int s = 0; s < nstep; ++s) {
             char* step = b + (size_t)s * 3 * kBlockBytes;
-            launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, 32 * s, 1, ROW_NATURAL, K_NATURAL, 1.f, step, stream);
+            // u rows are packed times -log2(e) and W_out times -ln(2): the kernel then needs
+            // u' v / (1 + exp2(u')) with u' = -log2(e) u, one multiply less per element
+            launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, 32 * s, 1, ROW_NATURAL, K_NATURAL, -kLog2e, step, stream);
             launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, hid + 32 * s, 1, ROW_NATURAL, K_NATURAL, 1.f,
                                step + kBlockBytes, stream);
             // W_out[:, 32s .. 32s+31]: a 32-wide column slice of the [C, hid] matrix
             launch_pack_blocks(static_cast<const char*>(out_w) + (size_t)32 * s * wsz, w_dtype, C, 32, hid,
-                               0, 4, ROW_INTERLEAVE4, K_ACC, 1.f, step + 2 * kBlockBytes, stream);
+                               0, 4, ROW_INTERLEAVE4, K_ACC, -1.0f / kLog2e, step + 2 * kBlockBytes, stream);
         }
         float* ln = reinterpret_cast<float*>(b + (size_t)nstep * 3 * kBlockBytes);
         launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);

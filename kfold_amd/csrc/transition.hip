@@ -80,9 +80,11 @@ __global__ __launch_bounds__(TILE * 2, 3) void transition_kernel(
             u = mfma32(w0, xf[ks], u);
             g = mfma32(w1, xf[ks], g);
         }
-        // hidden = silu(u) * v ; lane = position, registers = 16 of the step's hidden channels
+        // hidden = silu(u) * v ; lane = position, registers = 16 of the step's hidden channels.
+        // The packed u rows carry a factor -log2(e) and W_out its inverse, so with
+        // u' = -log2(e) u:  silu(u) v = (-ln 2) u' v / (1 + exp2(u')).
 #pragma unroll
-        for (int v = 0; v < 16; ++v) u[v] = u[v] * g[v] * fast_rcp(1.0f + fast_exp2(-kLog2e * u[v]));
+        for (int v = 0; v < 16; ++v) u[v] = u[v] * g[v] * fast_rcp(1.0f + fast_exp2(u[v]));
         bf16x8 hf0, hf1;
         acc_to_frags(u, hf0, hf1);
         // second GEMM: out[pos][c] += hidden[pos][32 of this step] * W_out[c][those 32]
