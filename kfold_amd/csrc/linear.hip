@@ -1,8 +1,8 @@
 // Generic bf16 MFMA linear layers for the single (token) track and the pair-bias attention
 // projections:  Y = X W^T (+ bias) followed by a small epilogue.  X is either row-major bf16
-// or already in MFMA fragment order; W is a packed weight (pack.hip).  One wavefront computes
-// one 32 x 32 output tile with operands read straight from global memory / L2: these
-// problems are a few hundred rows, so no LDS staging is used.
+// or already in MFMA fragment order; W is a packed weight (pack.hip).  One workgroup computes
+// one 32 x 32 output tile, its 4 wavefronts splitting K, with operands read straight from
+// global memory / L2: these problems are a few hundred rows, so no LDS staging is used.
 //
 // Epilogues (reference lines in src/kfold/model):
 //   EPI_STORE    y = acc + bias
@@ -20,8 +20,11 @@ template <int EPI, bool AFRAG>
 __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
-    const int wb = blockIdx.y * 4 + wave;
-    if (wb >= p.nblk) return;
+    // The 4 wavefronts of a workgroup share one 32 x 32 output tile and split K between them in
+    // chunks of 8 k-steps (wavefront w takes chunks w, w+4, ...): these problems have few tiles
+    // and long K, so the serial chain of dependent operand loads is what costs.
+    __shared__ float red[3][2][64 * 16];
+    const int wb = blockIdx.y;
     const int a = blockIdx.x / p.nb, blk = blockIdx.x % p.nb;
     const int ksteps = p.K / 16;
     const bf16x8* __restrict__ W = static_cast<const bf16x8*>(p.W) + (size_t)wb * ksteps * 64 + lane;
@@ -65,21 +68,42 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
         }
     };
     const int nch = ksteps / CH;
-    if (nch > 0) load(0, xa, wa, va);
-    for (int c = 0; c < nch; c += 2) {
-        if (c + 1 < nch) load(c + 1, xb, wb2, vb);
+    const int mine = nch > wave ? (nch - wave + 3) / 4 : 0;          // chunks of this wavefront
+    auto chunk = [&](int i) { return wave + 4 * i; };
+    if (mine > 0) load(chunk(0), xa, wa, va);
+    for (int i = 0; i < mine; i += 2) {
+        if (i + 1 < mine) load(chunk(i + 1), xb, wb2, vb);
         compute(xa, wa, va);
-        if (c + 1 < nch) {
-            if (c + 2 < nch) load(c + 2, xa, wa, va);
+        if (i + 1 < mine) {
+            if (i + 2 < mine) load(chunk(i + 2), xa, wa, va);
             compute(xb, wb2, vb);
         }
     }
-    for (int ks = nch * CH; ks < ksteps; ++ks) {      // K not a multiple of 128
-        const bf16x8 x = afrag(ks);
-        const bf16x8 w = W[(size_t)ks * 64];
-        acc = W_IS_A ? mfma32(w, x, acc) : mfma32(x, w, acc);
-        if constexpr (TWO) acc2 = mfma32(x, W2[(size_t)ks * 64], acc2);
+    if (wave == 0) {
+        for (int ks = nch * CH; ks < ksteps; ++ks) {      // K not a multiple of 128
+            const bf16x8 x = afrag(ks);
+            const bf16x8 w = W[(size_t)ks * 64];
+            acc = W_IS_A ? mfma32(w, x, acc) : mfma32(x, w, acc);
+            if constexpr (TWO) acc2 = mfma32(x, W2[(size_t)ks * 64], acc2);
+        }
     }
+    // partial sums of wavefronts 1..3 -> LDS -> wavefront 0, which runs the epilogue
+    if (wave > 0) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            red[wave - 1][0][v * 64 + lane] = acc[v];
+            if constexpr (TWO) red[wave - 1][1][v * 64 + lane] = acc2[v];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            acc[v] += red[w][0][v * 64 + lane];
+            if constexpr (TWO) acc2[v] += red[w][1][v * 64 + lane];
+        }
 
     if constexpr (EPI == EPI_FRAG_CH || EPI == EPI_FRAG_POS) {
         const int h = wb / p.PB, pp = wb % p.PB;
@@ -132,7 +156,7 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
 
 int launch_linear(const LinearArgs& p, hipStream_t stream) {
     if (p.K % 16 || p.nb <= 0 || p.rows_a <= 0) return -1;
-    dim3 grid((unsigned)(p.rows_a * p.nb), (unsigned)((p.nblk + 3) / 4)), block(256);
+    dim3 grid((unsigned)(p.rows_a * p.nb), (unsigned)p.nblk), block(256);
 #define KFH_LIN(E, F) hipLaunchKernelGGL((linear_kernel<E, F>), grid, block, 0, stream, p)
     switch (p.epi) {
         case EPI_STORE: if (p.a_frag) KFH_LIN(EPI_STORE, true); else KFH_LIN(EPI_STORE, false); break;
