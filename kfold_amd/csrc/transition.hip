@@ -35,14 +35,6 @@ __global__ __launch_bounds__(TILE * 2, 3) void transition_kernel(
         const long long p = p0 + row;
         return p < M ? p * kC : -1;
     };
-    stage_ln_rows<IO, TILE, decltype(row_off), NT>(
-        smem, x, reinterpret_cast<const float*>(blob + ln_off), eps, tid, row_off);
-    __syncthreads();
-    bf16x8 xf[kKS];
-#pragma unroll
-    for (int ks = 0; ks < kKS; ++ks) xf[ks] = lds_frag(smem, wave * 32 + col, ks, half);
-    __syncthreads();
-
     const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob);
     constexpr int NPRE = (kStepBytes / 16 + NT - 1) / NT;
     u32x4 pre[NPRE];
@@ -51,13 +43,21 @@ __global__ __launch_bounds__(TILE * 2, 3) void transition_kernel(
         for (int i = 0; i < NPRE; ++i)
             if (i * NT + tid < kStepBytes / 16) pre[i] = wsrc[(size_t)s * (kStepBytes / 16) + i * NT + tid];
     };
+    prefetch(0);        // the first weight step travels while the rows are loaded and normalised
+    stage_ln_rows<IO, TILE, decltype(row_off), NT>(
+        smem, x, reinterpret_cast<const float*>(blob + ln_off), eps, tid, row_off);
+    __syncthreads();
+    bf16x8 xf[kKS];
+#pragma unroll
+    for (int ks = 0; ks < kKS; ++ks) xf[ks] = lds_frag(smem, wave * 32 + col, ks, half);
+    __syncthreads();
+
     auto commit = [&](int s) {
 #pragma unroll
         for (int i = 0; i < NPRE; ++i)
             if (i * NT + tid < kStepBytes / 16)
                 reinterpret_cast<u32x4*>(smem + (s & 1) * kStepBytes)[i * NT + tid] = pre[i];
     };
-    prefetch(0);
     commit(0);
     __syncthreads();
 

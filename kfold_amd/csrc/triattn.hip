@@ -53,6 +53,14 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
         const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
         return (long long)(pos * kC);
     };
+    const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTaProjOff);
+    constexpr int NPRE = 1024 / NT;
+    u32x4 pre[NPRE];
+    auto prefetch = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < NPRE; ++i) pre[i] = wsrc[s * 1024 + i * NT + tid];
+    };
+    prefetch(0);        // the first weight step travels while the rows are loaded and normalised
     stage_ln_rows<IO, kTileA, decltype(row_off), NT>(
         smem, x, reinterpret_cast<const float*>(blob + kTaLnOff), eps, tid, row_off);
     __syncthreads();
@@ -81,13 +89,6 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
     //   0..3  { q_h , k_h }   both with channels as accumulator rows (weights = A operand)
     //   4..7  { g_h , v_h }   g_h like q; v_h with positions as rows (activations = A operand)
     //   8     { pair bias, - } rows 0..3 of the block are the 4 heads
-    const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTaProjOff);
-    constexpr int NPRE = 1024 / NT;
-    u32x4 pre[NPRE];
-    auto prefetch = [&](int s) {
-#pragma unroll
-        for (int i = 0; i < NPRE; ++i) pre[i] = wsrc[s * 1024 + i * NT + tid];
-    };
     auto commit = [&](int s) {
 #pragma unroll
         for (int i = 0; i < NPRE; ++i)
@@ -102,7 +103,6 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
         dst[frag_index(a, h, blk0 + pb, 0, nb, lane)] = f0;
         dst[frag_index(a, h, blk0 + pb, 1, nb, lane)] = f1;
     };
-    prefetch(0);
     commit(0);
     __syncthreads();
 

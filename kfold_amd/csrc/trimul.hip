@@ -53,6 +53,14 @@ __global__ __launch_bounds__(TILE * 2, 4) void trimul_in_kernel(
         const size_t pos = incoming ? (size_t)t * N + line : (size_t)line * N + t;
         return (long long)(pos * kC);
     };
+    const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTmInOff);
+    constexpr int NPRE = 1024 / NT;
+    u32x4 pre[NPRE];
+    auto prefetch = [&](int s) {
+#pragma unroll
+        for (int i = 0; i < NPRE; ++i) pre[i] = wsrc[s * 1024 + i * NT + tid];
+    };
+    prefetch(0);        // the first weight step travels while the rows are loaded and normalised
     stage_ln_rows<IO, TILE, decltype(row_off), NT>(
         smem, z, reinterpret_cast<const float*>(blob + kTmLnOff), eps, tid, row_off);
     __syncthreads();
@@ -76,13 +84,6 @@ __global__ __launch_bounds__(TILE * 2, 4) void trimul_in_kernel(
     // After the gate steps the fragments of masked positions are zeroed, which makes
     // ab = p * sigmoid(g) * mask come out as exact zeros without a multiply (no bias terms).
     constexpr int NSTEP = 10;
-    const u32x4* wsrc = reinterpret_cast<const u32x4*>(blob + kTmInOff);
-    constexpr int NPRE = 1024 / NT;
-    u32x4 pre[NPRE];
-    auto prefetch = [&](int s) {
-#pragma unroll
-        for (int i = 0; i < NPRE; ++i) pre[i] = wsrc[s * 1024 + i * NT + tid];
-    };
     auto commit = [&](int s) {
 #pragma unroll
         for (int i = 0; i < NPRE; ++i)
@@ -91,7 +92,6 @@ __global__ __launch_bounds__(TILE * 2, 4) void trimul_in_kernel(
     auto wfrag = [&](int s, int blk, int ks) {
         return *reinterpret_cast<const bf16x8*>(smem + (s & 1) * 16384 + blk * 8192 + ks * 1024 + lane * 16);
     };
-    prefetch(0);
     commit(0);
     __syncthreads();
 
