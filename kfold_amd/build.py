@@ -24,7 +24,7 @@ FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-unused-command-line-argument",
-] + os.environ.get("KFH_EXTRA_FLAGS", "").split()
+]
 
 
 def sources() -> list[Path]:

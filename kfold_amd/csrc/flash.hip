@@ -21,8 +21,8 @@
 // exponent needs no subtraction), then the scores.  A lane then owns 16 keys of one query: the
 // row max and row sum need one cross-half exchange, and exp2(S - m) rounded to bf16 is
 // already the B operand of O^T[d][query] += V^T[d][key] P^T[key][query].  m only moves when
-// a logit exceeds it by 2^8 (lazy rescale); it is kept bf16-representable so the MFMA
-// subtracts it exactly.
+// a logit exceeds it by 2^8 (lazy rescale, exact path) or a lane's partial row sum exceeds
+// 2^40 (max-free path); it is kept bf16-representable so the MFMA subtracts it exactly.
 //
 // Two kernels share that tile code:
 //   flash_strip_kernel  (triangle attention, N <= 1216): a workgroup owns one head, two query
@@ -35,8 +35,6 @@
 // Masking follows the reference's finite -1e9 semantics: in a row with a valid key, masked
 // keys get probability exactly 0; in a row with no valid key all real keys get the same
 // logit (q.k + bias is absorbed by -1e9 in fp32), i.e. uniform attention.
-#include <cstdlib>
-
 #include "kernels.hpp"
 
 namespace kfh {
@@ -128,29 +126,6 @@ __device__ __forceinline__ void rescale(f32x16& s, float mx, float& m, float& l,
         for (int v = 0; v < 16; ++v) o[d][v] *= alpha;
 #pragma unroll
     for (int v = 0; v < 16; ++v) s[v] -= delta;
-}
-
-// Sum of 16 bf16 values held as 8 packed dwords: two chains of v_dot2c_f32_bf16 against a
-// vector of ones, fp32 accumulation.  Written as one inline-assembly block because (a) with
-// hipcc 7.2 the __builtin_amdgcn_fdot2_f32_bf16 form of this chain was compiled into four dot
-// products of the same source register, and (b) a DOT result needs three wait states before
-// a non-DOT VALU instruction may read it, which the compiler cannot know for inline
-// assembly: the trailing s_nop provides them.
-__device__ __forceinline__ float sum16_bf16(const u32x4& a, const u32x4& b) {
-    float t0 = 0.f, t1 = 0.f;
-    const uint32_t ones = 0x3f803f80u;
-    asm("v_dot2c_f32_bf16 %0, %2, %10\n\t"
-        "v_dot2c_f32_bf16 %1, %6, %10\n\t"
-        "v_dot2c_f32_bf16 %0, %3, %10\n\t"
-        "v_dot2c_f32_bf16 %1, %7, %10\n\t"
-        "v_dot2c_f32_bf16 %0, %4, %10\n\t"
-        "v_dot2c_f32_bf16 %1, %8, %10\n\t"
-        "v_dot2c_f32_bf16 %0, %5, %10\n\t"
-        "v_dot2c_f32_bf16 %1, %9, %10\n\t"
-        "s_nop 2"
-        : "+v"(t0), "+v"(t1)
-        : "v"(a[0]), "v"(a[1]), "v"(a[2]), "v"(a[3]), "v"(b[0]), "v"(b[1]), "v"(b[2]), "v"(b[3]), "v"(ones));
-    return t0 + t1;
 }
 
 // p = bf16(exp2(s)) as the two B-operand fragments of the PV product; returns this lane's
