@@ -87,3 +87,29 @@ def test_state_dict_names_match_reference_names():
     assert set(ta) == {"layer_norm.weight", "layer_norm.bias", "linear.weight", "mha.linear_q.weight",
                        "mha.linear_k.weight", "mha.linear_v.weight", "mha.linear_o.weight",
                        "mha.linear_g.weight"}
+
+
+def test_no_cpu_fallback_in_the_product_path():
+    """The modules never compute on the host: CPU tensors are refused, training mode is refused,
+    and nothing under kfold_amd imports the oracle."""
+    import torch
+
+    from kfold_amd import layers, primitives
+
+    x = torch.zeros(1, 8, 8, 128)
+    m = torch.ones(1, 8, 8)
+    for mod in (primitives.TriangleMultiplicationOutgoing(128).eval(),
+                primitives.TriangleAttentionStartingNode(128, 4).eval()):
+        with pytest.raises((RuntimeError, ValueError)):
+            with torch.no_grad():
+                mod(x, m)
+    with pytest.raises((RuntimeError, ValueError)):
+        with torch.no_grad():
+            layers.Transition(128, 2).eval()(x)
+    for path in (ROOT / "kfold_amd").rglob("*.py"):
+        text = path.read_text()
+        assert "import oracle" not in text and "from oracle" not in text, path
+    for name in ("bench.py",):
+        # the benchmark may only use the oracle for its cpu_baseline leg
+        text = (ROOT / name).read_text()
+        assert text.count("from oracle") == 1 and "def cpu_baseline" in text
