@@ -66,7 +66,7 @@ def test_triattn_general_mask_none_mask_f32_io(starting):
 
 @pytest.mark.parametrize("starting", [True, False])
 def test_triattn_config3_n512(starting):
-    """BASELINE config 3: N=512, key mask zeroing the last 64 tokens, bf16."""
+    """Benchmark config 3: N=512, key mask zeroing the last 64 tokens, bf16."""
     print(f"case triattn config3 starting={starting}", flush=True)
     ref, hip = _modules(starting)
     x, _, pm = synthetic.pair_inputs(512, 128, 64, seed=0)

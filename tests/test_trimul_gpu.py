@@ -61,7 +61,7 @@ def test_trimul_general_mask_and_f32_io(direction):
 
 @pytest.mark.parametrize("direction", ["outgoing", "incoming"])
 def test_trimul_config2_n384(direction):
-    """BASELINE config 2: N=384, last 38 tokens padded, bf16."""
+    """Benchmark config 2: N=384, last 38 tokens padded, bf16."""
     print(f"case trimul config2 {direction}", flush=True)
     ref, hip = _modules(direction)
     z, _, pm = synthetic.pair_inputs(384, 128, 38, seed=0)
