@@ -31,7 +31,7 @@ CAL_COPY_BYTES = 256 << 20     # size of the counter-calibration copy
 # HBM bytes per launch of the attention kernel at N=768 (FETCH_SIZE + WRITE_SIZE, each scaled by
 # the calibration copy's reading in the same run); the counter runs are summarised in
 # profiles/hot_path_kernels_n768_hbm_traffic.md.  None where no counter run exists.
-MEASURED_TRAFFIC_BYTES = {768: 851160183}
+MEASURED_TRAFFIC_BYTES = {768: 851100477}
 
 
 def block_flops(n: int) -> dict:
