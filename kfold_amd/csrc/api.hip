@@ -203,10 +203,11 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
                 launch_fill_zero(ws.biast + (((size_t)h * sz.nb + (sz.nb - 1)) * sz.nb) * kBiasTileElems,
                                  (size_t)sz.nb * 2048, stream);
         }
-        launch_triattn(static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N,
-                       static_cast<const char*>(blob), ws,
-                       residual ? static_cast<const char*>(residual) + off : nullptr,
-                       static_cast<char*>(out) + off, N, ending, eps, stages, stream);
+        const int rc = launch_triattn(static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N,
+                                      static_cast<const char*>(blob), ws,
+                                      residual ? static_cast<const char*>(residual) + off : nullptr,
+                                      static_cast<char*>(out) + off, N, ending, eps, stages, stream);
+        if (rc) return fail(KFH_EHIP, "triattn_forward: attention kernel launch failed (%d)", rc);
     }
     return check_launch("triattn_forward");
 }

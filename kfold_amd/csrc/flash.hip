@@ -35,6 +35,8 @@
 // Masking follows the reference's finite -1e9 semantics: in a row with a valid key, masked
 // keys get probability exactly 0; in a row with no valid key all real keys get the same
 // logit (q.k + bias is absorbed by -1e9 in fp32), i.e. uniform attention.
+#include <atomic>
+
 #include "kernels.hpp"
 
 namespace kfh {
@@ -631,24 +633,26 @@ static int launch_staged(FlashArgs p, int head_dim_pad, hipStream_t stream) {
 
 static int launch_strip(FlashArgs p, hipStream_t stream) {
     const size_t lds_bytes = (size_t)p.nb * 4096 + kStripWaves * 64;
-    static bool attr_set = false;
-    if (!attr_set) {
+    // per-device launch state (a process may drive several GPUs; the writes are idempotent, so
+    // concurrent first calls are harmless)
+    constexpr int kMaxDevices = 64;
+    static std::atomic<int> cu_count[kMaxDevices];      // 0 = not queried yet
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -2;
+    int n_cu = cu_count[dev].load(std::memory_order_relaxed);
+    if (n_cu == 0) {
+        // the strip needs more dynamic LDS than the default limit: raise it once per device
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(flash_strip_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize,
                                 kStripMaxBlocks * 4096 + kStripWaves * 64) != hipSuccess)
             return -2;
-        attr_set = true;
+        if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0)
+            n_cu = 256;
+        cu_count[dev].store(n_cu, std::memory_order_relaxed);
     }
     p.qgroups = (p.nb + 1) / 2;                                    // query-block pairs
     // rows per workgroup: a multiple of the wavefront count; one workgroup per CU is resident,
     // so pick the split whose number of full-chip rounds times rows per round is smallest
-    static int n_cu = 0;
-    if (n_cu == 0) {
-        int dev = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0)
-            n_cu = 256;
-    }
     int per = kStripWaves;
     long long best = -1;
     for (int cand = kStripWaves; cand <= kStripWaves * 8; cand += kStripWaves) {

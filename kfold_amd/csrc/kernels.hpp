@@ -75,7 +75,8 @@ struct FlashArgs {
 int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
 
 void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream);
-void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
+// returns 0, or the non-zero status of the attention launch (shape not built, HIP error)
+int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
                     float eps, int stages, hipStream_t stream);
 

@@ -266,7 +266,7 @@ __global__ __launch_bounds__(512, 3) void triattn_out_kernel(
 }
 
 // ------------------------------------------------------------------------------------------
-void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
+int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
                     float eps, int stages, hipStream_t stream) {
     const int nb = (N + 31) / 32;
@@ -289,8 +289,11 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
     fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = gf; fa.of = of;
     fa.biast = ws.biast; fa.codes = ws.codes;
     fa.nrows = N; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
-    if (stages & KFH_STAGE_CORE) launch_flash(fa, 32, stream);
-    if (!(stages & KFH_STAGE_OUT)) return;
+    if (stages & KFH_STAGE_CORE) {
+        const int rc = launch_flash(fa, 32, stream);
+        if (rc) return rc;
+    }
+    if (!(stages & KFH_STAGE_OUT)) return 0;
 
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, dim3(512), 0, stream, of, blob,
@@ -298,6 +301,7 @@ void launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char
     else
         hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, dim3(512), 0, stream, of, blob,
                            residual, out, N, nb, ending);
+    return 0;
 }
 
 }  // namespace kfh
