@@ -321,12 +321,26 @@ class SelfAttentionPairBias(nn.Module):
 # ---------------------------------------------------------------------------
 # blocks
 # ---------------------------------------------------------------------------
+def _stream_add_(x: torch.Tensor, update: torch.Tensor, stream_dtype) -> None:
+    """``x += update`` in place (primitives/utils.py:47-48).  With ``stream_dtype`` set the sum is
+    rounded to that dtype (and kept in the tensor's own dtype): the values a residual stream
+    stored in ``stream_dtype`` holds after the add, as under the reference's bf16 autocast
+    (inference/runner.py:565-571) where ``z`` itself is a bf16 tensor."""
+    x.add_(update)
+    if stream_dtype is not None:
+        x.copy_(x.to(stream_dtype))
+
+
 class PairformerBlock(nn.Module):
-    """model/modules/apo_module.py:107-172, eval mode (dropout is the identity)."""
+    """model/modules/apo_module.py:107-172, eval mode (dropout is the identity).
+
+    ``stream_dtype``: round the residual stream to this dtype after every in-place add
+    (None = the all-fp32 oracle).  The arithmetic of every op stays fp32 either way."""
 
     def __init__(self, channel_z: int = 128, num_tri_heads: int = 4,
-                 row_chunk: int | None = None):
+                 row_chunk: int | None = None, stream_dtype: torch.dtype | None = None):
         super().__init__()
+        self.stream_dtype = stream_dtype
         self.tri_mul_out = TriangleMultiplicationOutgoing(channel_z)
         self.tri_mul_in = TriangleMultiplicationIncoming(channel_z)
         self.tri_att_start = TriangleAttentionStartingNode(channel_z, num_tri_heads,
@@ -337,12 +351,32 @@ class PairformerBlock(nn.Module):
 
     def forward(self, z: torch.Tensor, pair_mask: torch.Tensor) -> torch.Tensor:
         # in eval mode the adds mutate the caller's tensor (primitives/utils.py:47-48)
-        z.add_(self.tri_mul_out(z, pair_mask))
-        z.add_(self.tri_mul_in(z, pair_mask))
-        z.add_(self.tri_att_start(z, pair_mask))
-        z.add_(self.tri_att_end(z, pair_mask))
-        z.add_(self.transition_z(z))
+        sd = self.stream_dtype
+        _stream_add_(z, self.tri_mul_out(z, pair_mask), sd)
+        _stream_add_(z, self.tri_mul_in(z, pair_mask), sd)
+        _stream_add_(z, self.tri_att_start(z, pair_mask), sd)
+        _stream_add_(z, self.tri_att_end(z, pair_mask), sd)
+        _stream_add_(z, self.transition_z(z), sd)
         return z * pair_mask[..., None]
+
+
+class TriangularBlock(nn.Module):
+    """model/modules/tri_stack.py:96-151, eval mode: tri-mul out, tri-mul in, transition x4,
+    every update added in place (:138-150); no triangle attention and no final mask."""
+
+    def __init__(self, channel_z: int = 128, stream_dtype: torch.dtype | None = None):
+        super().__init__()
+        self.stream_dtype = stream_dtype
+        self.tri_mul_out = TriangleMultiplicationOutgoing(channel_z)
+        self.tri_mul_in = TriangleMultiplicationIncoming(channel_z)
+        self.transition_z = Transition(channel_z, expansion_factor=4)
+
+    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor) -> torch.Tensor:
+        sd = self.stream_dtype
+        _stream_add_(z, self.tri_mul_out(z, pair_mask), sd)
+        _stream_add_(z, self.tri_mul_in(z, pair_mask), sd)
+        _stream_add_(z, self.transition_z(z), sd)
+        return z
 
 
 class PairSingleBlock(nn.Module):
@@ -356,9 +390,12 @@ class PairSingleBlock(nn.Module):
     """
 
     def __init__(self, channel_s: int = 384, channel_z: int = 128, num_heads: int = 16,
-                 num_tri_heads: int = 4, row_chunk: int | None = None):
+                 num_tri_heads: int = 4, row_chunk: int | None = None,
+                 stream_dtype: torch.dtype | None = None):
         super().__init__()
-        self.pair_block = PairformerBlock(channel_z, num_tri_heads, row_chunk=row_chunk)
+        self.stream_dtype = stream_dtype
+        self.pair_block = PairformerBlock(channel_z, num_tri_heads, row_chunk=row_chunk,
+                                          stream_dtype=stream_dtype)
         self.layernorm_z = LayerNorm(channel_z)
         self.linear_pair_bias = LinearNoBias(channel_z, num_heads)
         self.attention = SelfAttentionPairBias(channel_s, num_heads, None, call_site="confidence")
@@ -367,8 +404,8 @@ class PairSingleBlock(nn.Module):
     def forward(self, z, s, pair_mask, mask):
         z = self.pair_block(z, pair_mask)
         pair_bias = self.linear_pair_bias(self.layernorm_z(z)).movedim(-1, -3)
-        s.add_(self.attention(s, None, pair_bias, mask))
-        s.add_(self.transition(s))
+        _stream_add_(s, self.attention(s, None, pair_bias, mask), self.stream_dtype)
+        _stream_add_(s, self.transition(s), self.stream_dtype)
         return z, s
 
 
@@ -376,10 +413,11 @@ class PairformerTrunk(nn.Module):
     """A stack of ``PairSingleBlock`` (plain loop at inference, utils/checkpointing.py:85-86)."""
 
     def __init__(self, num_blocks: int, channel_s: int = 384, channel_z: int = 128,
-                 num_heads: int = 16, num_tri_heads: int = 4, row_chunk: int | None = None):
+                 num_heads: int = 16, num_tri_heads: int = 4, row_chunk: int | None = None,
+                 stream_dtype: torch.dtype | None = None):
         super().__init__()
         self.blocks = nn.ModuleList(
-            PairSingleBlock(channel_s, channel_z, num_heads, num_tri_heads, row_chunk)
+            PairSingleBlock(channel_s, channel_z, num_heads, num_tri_heads, row_chunk, stream_dtype)
             for _ in range(num_blocks))
 
     def forward(self, z, s, pair_mask, mask):

@@ -1,44 +1,92 @@
-"""HIP Pairformer block / trunk vs the fp32 oracle."""
+"""HIP Pairformer block / trunk vs the oracle.
+
+A bf16 residual stream is rounded after each in-place update, which alone moves ``z`` away
+from the all-fp32 oracle by more than the north-star limits (|z| ~ N(0,1) reaches 4-6, where
+bf16 steps are 2^-5).  The block tests therefore separate the two sources of error:
+
+* stage by stage ("teacher forced"): every in-place update of the HIP block is compared, at
+  the unscaled limits, with the fp32 oracle op applied to the very same bf16 input;
+* end to end against the oracle run with a bf16-rounded stream, with the all-fp32 oracle as
+  control (see ``tests.util.assert_stream_close``);
+* with fp32 activations at the boundary (no storage rounding) the whole block meets the
+  unscaled limits against the all-fp32 oracle.
+"""
 
 import pytest
 import torch
 
 from kfold_amd import synthetic
-from tests.util import assert_close
+from tests.util import assert_close, assert_stream_close
 
 pytestmark = pytest.mark.gpu
 
 DEV = "cuda:0"
 
 
-def _blocks(num=1, seed=0, std=0.02):
+def _blocks(num=1, seed=0, std=0.02, row_chunk=32):
     from kfold_amd import modules as M
     from oracle import torch_path as O
 
-    ref = O.PairformerTrunk(num, row_chunk=32).eval()
+    ref = O.PairformerTrunk(num, row_chunk=row_chunk).eval()
     synthetic.init_weights_(ref, seed, std=std)
+    stream = O.PairformerTrunk(num, row_chunk=row_chunk, stream_dtype=torch.bfloat16).eval()
+    stream.load_state_dict(ref.state_dict())
     hip = M.PairformerTrunk(num).eval()
     hip.load_state_dict(ref.state_dict())
-    return ref, hip.to(DEV)
+    return ref, stream, hip.to(DEV)
+
+
+def pair_stages(ref_block, hip_block, pm, pm_dev):
+    """(name, oracle update fn, HIP in-place fn) for the five updates of the pair track; the last
+    one carries the block's final mask."""
+    from kfold_amd import modules as M
+    from kfold_amd.layers.transition import hip_transition
+
+    rb, hb = ref_block.pair_block, hip_block.pair_block
+    pmf = pm.float()
+    return [
+        ("tri_mul_out", lambda x: x + rb.tri_mul_out(x, pmf),
+         lambda x: M._trimul_inplace(hb.tri_mul_out, x, pm_dev)),
+        ("tri_mul_in", lambda x: x + rb.tri_mul_in(x, pmf),
+         lambda x: M._trimul_inplace(hb.tri_mul_in, x, pm_dev)),
+        ("tri_att_start", lambda x: x + rb.tri_att_start(x, pmf),
+         lambda x: M._triattn_inplace(hb.tri_att_start, x, pm_dev)),
+        ("tri_att_end", lambda x: x + rb.tri_att_end(x, pmf),
+         lambda x: M._triattn_inplace(hb.tri_att_end, x, pm_dev)),
+        ("transition_z + mask", lambda x: (x + rb.transition_z(x)) * pmf[..., None],
+         lambda x: hip_transition(hb.transition_z, x, residual=x, mask=pm_dev, out=x)),
+    ]
+
+
+def check_stagewise(ref_block, hip_block, z_dev, pm, what):
+    """Walk the pair track on the HIP stream ``z_dev`` (in place); before each update the oracle
+    op is evaluated in fp32 on a copy of the stream's current values."""
+    out = {}
+    with torch.no_grad():
+        for name, ref_fn, hip_fn in pair_stages(ref_block, hip_block, pm, pm.to(z_dev.device)):
+            want = ref_fn(z_dev.float().cpu())
+            hip_fn(z_dev)
+            out[name] = assert_close(z_dev, want, f"{what} stage {name}", rel_fro=None)
+    return out
 
 
 @pytest.mark.parametrize("n,frac", [(64, 0.0), (100, 0.15)])
 def test_block_parity_and_masked_zero(n, frac):
     """Config 1 shape (N=64, all-ones mask) and a padded odd size, one block, bf16."""
     print(f"case block n={n} pad={frac}", flush=True)
-    ref, hip = _blocks(1)
+    ref, stream, hip = _blocks(1)
     z, tok, pm = synthetic.pair_inputs(n, 128, synthetic.n_pad_for(n, frac), seed=0)
     s = synthetic.single_inputs(n, 384, seed=1)
     zb, sb = z.bfloat16(), s.bfloat16()
     with torch.no_grad():
         zw, sw = ref(zb.float(), sb.float(), pm.float(), tok.float())
+        zs, ss = stream(zb.float(), sb.float(), pm.float(), tok.float())
         zin, sin = zb.to(DEV), sb.to(DEV)
         zg, sg = hip(zin, sin, pm.to(DEV), tok.to(DEV))
-    # The residual stream |z| ~ N(0,1) is stored in bf16 and rounded after each of the 5
-    # in-place updates (as a bf16 z would be by the reference's own z.add_), so the absolute
-    # error scales with |z|; the fp32-io test below holds the unscaled tolerances.
-    assert_close(zg, zw, "block z", rel_fro=8e-3, auto_scale=True)
-    assert_close(sg, sw, "block s", rel_fro=8e-3, auto_scale=True)
+    print(assert_stream_close(zg, zs, zw, "block z"), flush=True)
+    print(assert_stream_close(sg, ss, sw, "block s"), flush=True)
+    # every update on its own, unscaled limits
+    check_stagewise(ref.blocks[0], hip.blocks[0], zb.to(DEV), pm, f"block n={n}")
     # masked positions are bit-exact zero
     assert (zg.cpu()[~pm] == 0).all()
     # in place like the reference's eval-mode adds
@@ -57,10 +105,8 @@ def test_block_parity_and_masked_zero(n, frac):
 def test_block_f32_io_fresh_output_and_update_size():
     """fp32 activations at the boundary (config 1 dtype); the update itself, not only the
     residual stream, must match."""
-    from kfold_amd import modules as M
-
     print("case block f32", flush=True)
-    ref, hip = _blocks(1, seed=2, std=0.05)
+    ref, _, hip = _blocks(1, seed=2, std=0.05)
     n = 48
     z, tok, pm = synthetic.pair_inputs(n, 128, 6, seed=3)
     s = synthetic.single_inputs(n, 384, seed=4)
@@ -78,16 +124,75 @@ def test_block_f32_io_fresh_output_and_update_size():
     assert (zg.cpu()[~pm] == 0).all()
 
 
+def test_config1_block_f32_io_all_ones_mask():
+    """Config 1 exactly: N=64, fp32 z and s at the boundary, all-ones masks, std-0.02 weights."""
+    print("case config 1", flush=True)
+    ref, _, hip = _blocks(1)
+    z, tok, pm = synthetic.pair_inputs(64, 128, 0, seed=0)
+    s = synthetic.single_inputs(64, 384, seed=1)
+    with torch.no_grad():
+        zw, sw = ref(z.clone(), s.clone(), pm.float(), tok.float())
+        zg, sg = hip(z.to(DEV), s.to(DEV), pm.to(DEV), tok.to(DEV))
+    print(assert_close(zg, zw, "config 1 z", rel_fro=3e-3), flush=True)
+    print(assert_close(sg, sw, "config 1 s", rel_fro=3e-3), flush=True)
+
+
 def test_trunk_three_blocks():
     print("case trunk x3", flush=True)
-    ref, hip = _blocks(3, seed=5)
+    ref, stream, hip = _blocks(3, seed=5)
     n = 72
     z, tok, pm = synthetic.pair_inputs(n, 128, 9, seed=6)
     s = synthetic.single_inputs(n, 384, seed=7)
     zb, sb = z.bfloat16(), s.bfloat16()
     with torch.no_grad():
         zw, sw = ref(zb.float(), sb.float(), pm.float(), tok.float())
+        zs, ss = stream(zb.float(), sb.float(), pm.float(), tok.float())
         zg, sg = hip(zb.to(DEV), sb.to(DEV), pm.to(DEV), tok.to(DEV))
-    assert_close(zg, zw, "trunk z", rel_fro=1.5e-2, auto_scale=True)
-    assert_close(sg, sw, "trunk s", rel_fro=1.5e-2, auto_scale=True)
+    print(assert_stream_close(zg, zs, zw, "trunk z", max_flip_frac=2e-3, max_ulps=8), flush=True)
+    print(assert_stream_close(sg, ss, sw, "trunk s", max_flip_frac=2e-3, max_ulps=8), flush=True)
     assert (zg.cpu()[~pm] == 0).all()
+    # the same three blocks with an fp32 stream: no storage rounding, unscaled limits end to end
+    with torch.no_grad():
+        zf, sf = hip(zb.float().to(DEV), sb.float().to(DEV), pm.to(DEV), tok.to(DEV))
+    print(assert_close(zf, zw, "trunk z (fp32 stream)", rel_fro=8e-3), flush=True)
+    print(assert_close(sf, sw, "trunk s (fp32 stream)", rel_fro=8e-3), flush=True)
+
+
+def test_triangular_block():
+    """The shipping trunk block (tri-mul out, tri-mul in, transition x4, no final mask) at
+    c_z = 128: bf16 stream stage by stage, fp32 stream end to end."""
+    from kfold_amd import modules as M
+    from kfold_amd.layers.transition import hip_transition
+    from oracle import torch_path as O
+
+    print("case triangular block", flush=True)
+    ref = O.TriangularBlock(128).eval()
+    synthetic.init_weights_(ref, 11)
+    hip = M.TriangularBlock(128).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    n = 90
+    z, _, pm = synthetic.pair_inputs(n, 128, 11, seed=12)
+    zb = z.bfloat16()
+    with torch.no_grad():
+        zw = ref(zb.float(), pm.float())
+        zin = zb.float().to(DEV)
+        zg = hip(zin, pm.to(DEV))
+        assert zg.data_ptr() == zin.data_ptr()           # in place, like the reference in eval mode
+        print(assert_close(zg, zw, "triangular block (fp32 stream)", rel_fro=5e-3), flush=True)
+        # padded positions are NOT zeroed by this block (no final mask): they hold z + transition(z)
+        assert (zg.cpu()[~pm].abs().sum() > 0)
+        # bf16 stream, each update against the oracle op on the same input
+        zd = zb.to(DEV)
+        pmd, pmf = pm.to(DEV), pm.float()
+        stages = [
+            (lambda x: x + ref.tri_mul_out(x, pmf), lambda x: M._trimul_inplace(hip.tri_mul_out, x, pmd)),
+            (lambda x: x + ref.tri_mul_in(x, pmf), lambda x: M._trimul_inplace(hip.tri_mul_in, x, pmd)),
+            (lambda x: x + ref.transition_z(x), lambda x: hip_transition(hip.transition_z, x, residual=x, out=x)),
+        ]
+        for i, (rf, hf) in enumerate(stages):
+            want = rf(zd.float().cpu())
+            hf(zd)
+            assert_close(zd, want, f"triangular block stage {i}", rel_fro=None)
+        # the module call gives the same bits as the stage walk
+        assert torch.equal(hip(zb.to(DEV), pmd), zd)
