@@ -8,6 +8,13 @@
 
 using namespace kfh;
 
+// run a launch_* helper that reports an unsupported shape with a non-zero code
+#define KFH_TRY(call, what)                                                             \
+    do {                                                                                \
+        const int rc_ = (call);                                                         \
+        if (rc_ != 0) return fail(KFH_EUNSUPPORTED, "%s: shape not built (%d)", what, rc_); \
+    } while (0)
+
 namespace {
 
 // ---- blob / workspace layouts -------------------------------------------------------------
@@ -221,29 +228,29 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
 
     // 1. normalised input rows (bf16)
     if (!apply_norm) {
-        launch_rows_norm(a, io_dtype, nullptr, nullptr, xn, rows, C, 0, eps, stream);
+        KFH_TRY(launch_rows_norm(a, io_dtype, nullptr, nullptr, xn, rows, C, 0, eps, stream), "rows_norm");
     } else if (!Cs) {
-        launch_rows_norm(a, io_dtype, f32p(l.f_ln_g), f32p(l.f_ln_b), xn, rows, C, 1, eps, stream);
+        KFH_TRY(launch_rows_norm(a, io_dtype, f32p(l.f_ln_g), f32p(l.f_ln_b), xn, rows, C, 1, eps, stream), "rows_norm");
     } else {
         // AdaLN: sigmoid(W_g LN_s(s) + b_g) * LN(a) + W_b LN_s(s)
         const long long srows = s_per_sample ? rows : L;
         uint16_t* an = reinterpret_cast<uint16_t*>(ws + w.an);
         uint16_t* sn = reinterpret_cast<uint16_t*>(ws + w.sn);
         uint16_t* sraw = reinterpret_cast<uint16_t*>(ws + w.sraw);
-        launch_rows_norm(a, io_dtype, nullptr, nullptr, an, rows, C, 1, eps, stream);
-        launch_rows_norm(s_cond, io_dtype, f32p(l.f_lns_g), nullptr, sn, srows, Cs, 1, eps, stream);
-        launch_rows_norm(s_cond, io_dtype, nullptr, nullptr, sraw, srows, Cs, 0, eps, stream);
+        KFH_TRY(launch_rows_norm(a, io_dtype, nullptr, nullptr, an, rows, C, 1, eps, stream), "rows_norm");
+        KFH_TRY(launch_rows_norm(s_cond, io_dtype, f32p(l.f_lns_g), nullptr, sn, srows, Cs, 1, eps, stream), "rows_norm");
+        KFH_TRY(launch_rows_norm(s_cond, io_dtype, nullptr, nullptr, sraw, srows, Cs, 0, eps, stream), "rows_norm");
         LinearArgs p = plain(sn, Cs, L, Cs, b + l.w_adag, C);
         p.rows_a = S; p.a_shared = !s_per_sample;
         p.W2 = b + l.w_adab; p.bias = f32p(l.f_adag_b);
         p.aux = an; p.aux_dtype = KFH_BF16; p.ld_aux = C;
         p.out = xn; p.out_dtype = KFH_BF16; p.ldo = C; p.epi = EPI_ADALN;
-        launch_linear(p, stream);
+        KFH_TRY(launch_linear(p, stream), "linear");
         // output gate sigmoid(W_ada s + b_ada) on the raw conditioning
         LinearArgs g = plain(sraw, Cs, srows, Cs, b + l.w_adaout, C);
         g.bias = f32p(l.f_adaout_b);
         g.out = ws + w.gate_out; g.out_dtype = KFH_BF16; g.ldo = C; g.epi = EPI_SIGMOID;
-        launch_linear(g, stream);
+        KFH_TRY(launch_linear(g, stream), "linear");
     }
 
     // 2. q (with bias, pre-scaled), k, gate, v projections into fragment order
@@ -253,15 +260,15 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
         p.epi = EPI_FRAG_CH;
         p.W = b + l.wq; p.bias = f32p(l.f_bq); p.bias_scale = kLog2e / sqrtf((float)l.Dh);
         p.out = ws + w.qf;
-        launch_linear(p, stream);
+        KFH_TRY(launch_linear(p, stream), "linear");
         p.bias = nullptr;
         p.W = b + l.wk; p.out = ws + w.kf;
-        launch_linear(p, stream);
+        KFH_TRY(launch_linear(p, stream), "linear");
         p.W = b + l.wg; p.out = ws + w.gf; p.sigmoid = 1;
-        launch_linear(p, stream);
+        KFH_TRY(launch_linear(p, stream), "linear");
         p.sigmoid = 0; p.epi = EPI_FRAG_POS;
         p.W = b + l.wv; p.out = ws + w.vf;
-        launch_linear(p, stream);
+        KFH_TRY(launch_linear(p, stream), "linear");
     }
 
     // 3. key codes, attention
@@ -283,7 +290,7 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
         if (cond) { p.gate = reinterpret_cast<const uint16_t*>(ws + w.gate_out); p.ld_gate = C; p.gate_shared = !s_per_sample; }
         if (residual) { p.aux = residual; p.aux_dtype = io_dtype; p.ld_aux = C; }
         p.out = out; p.out_dtype = io_dtype; p.ldo = C;
-        launch_linear(p, stream);
+        KFH_TRY(launch_linear(p, stream), "linear");
     }
     return check_launch("apb_forward");
 }
@@ -353,7 +360,8 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* b = static_cast<const char*>(blob);
     if (C == kC && (expansion == 2 || expansion == 4)) {
-        launch_pair_transition(x, io_dtype, b, expansion, residual, mask, out, rows, eps, stream);
+        KFH_TRY(launch_pair_transition(x, io_dtype, b, expansion, residual, mask, out, rows, eps, stream),
+                "pair transition");
         return check_launch("transition_forward");
     }
     if (mask) return fail(KFH_EUNSUPPORTED, "transition_forward: the row mask is built for C=128 only");
@@ -366,15 +374,15 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
     uint16_t* xn = reinterpret_cast<uint16_t*>(ws);
     uint16_t* hid = reinterpret_cast<uint16_t*>(ws + align_up((size_t)rows * C * 2));
     const float* ln = reinterpret_cast<const float*>(b + l.f_ln);
-    launch_rows_norm(x, io_dtype, ln, ln + C, xn, rows, C, 1, eps, stream);
+    KFH_TRY(launch_rows_norm(x, io_dtype, ln, ln + C, xn, rows, C, 1, eps, stream), "rows_norm");
     LinearArgs p = plain(xn, C, rows, C, b + l.wu, l.hid);
     p.W2 = b + l.wv; p.out = hid; p.out_dtype = KFH_BF16; p.ldo = l.hid; p.epi = EPI_SWIGLU;
-    launch_linear(p, stream);
+    KFH_TRY(launch_linear(p, stream), "linear");
     LinearArgs q = plain(hid, l.hid, rows, l.hid, b + l.wo, C);
     q.epi = EPI_RESID;
     if (residual) { q.aux = residual; q.aux_dtype = io_dtype; q.ld_aux = C; }
     q.out = out; q.out_dtype = io_dtype; q.ldo = C;
-    launch_linear(q, stream);
+    KFH_TRY(launch_linear(q, stream), "linear");
     return check_launch("transition_forward");
 }
 

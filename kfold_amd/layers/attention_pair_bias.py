@@ -17,7 +17,7 @@ import torch
 from torch import nn
 
 from .. import ops
-from ..primitives._common import cache_key, cached_blob, check_inference
+from ..primitives._common import cache_key, cached_blob, check_inf, check_inference
 from ..primitives.layers import LayerNorm, Linear, LinearNoBias
 
 
@@ -41,6 +41,17 @@ def _cond_channels(module: nn.Module) -> int:
     return 0
 
 
+def norm_eps(module: nn.Module) -> float:
+    """The one LayerNorm epsilon the fused entry point takes: ``layernorm_a.eps``, or for the
+    conditioned module the common value of AdaLN's two LayerNorms."""
+    if getattr(module, "use_single_conditioning", False):
+        ea, es = module.adaln_a.layernorm_a.eps, module.adaln_a.layernorm_s.eps
+        if ea != es:
+            raise NotImplementedError(f"hip AdaLN: layernorm_a.eps ({ea}) != layernorm_s.eps ({es})")
+        return ea
+    return module.layernorm_a.eps if hasattr(module, "layernorm_a") else 1e-5
+
+
 def _flatten(t: torch.Tensor, keep: int, lead: torch.Size):
     """Flatten the leading dims of ``t`` (which broadcast against ``lead``) to 1 or prod(lead)."""
     tl = t.shape[:t.dim() - keep]
@@ -52,6 +63,7 @@ def _flatten(t: torch.Tensor, keep: int, lead: torch.Size):
 
 def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
     check_inference(a, "pair-bias attention")
+    check_inf(module)
     if module.linear_g.bias is not None or module.linear_out.bias is not None:
         raise NotImplementedError("hip pair-bias attention: gate / output projection biases")
     params = _parameters(module)
@@ -69,7 +81,7 @@ def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
         sf, _ = _flatten(s, 2, lead)
     tiles = ops.bias_tiles_from_dense(pb)
     out = ops.apb_forward(af, sf, tiles, mk, blob, H, Cs, apply_norm, per_sample and af.shape[0] > 1,
-                          eps=1e-5)
+                          eps=norm_eps(module))
     return out.reshape(a.shape).to(a.dtype)
 
 

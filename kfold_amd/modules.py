@@ -17,9 +17,9 @@ import torch
 from torch import nn
 
 from . import ops
-from .layers.attention_pair_bias import SelfAttentionPairBias, _cond_channels, _parameters
+from .layers.attention_pair_bias import SelfAttentionPairBias, _cond_channels, _parameters, norm_eps
 from .layers.transition import Transition, hip_transition
-from .primitives._common import cache_key, cached_blob, check_inference
+from .primitives._common import cache_key, cached_blob, check_inf, check_inference
 from .primitives.layers import LayerNorm, LinearNoBias
 from .primitives.triangle_attention import (
     TriangleAttentionEndingNode,
@@ -48,6 +48,7 @@ def _trimul_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None
 
 
 def _triattn_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None:
+    check_inf(mod)
     params = _ta_parameters(mod)
     blob = cached_blob(mod, "_hip_attention_cache", cache_key(params, z, torch.bfloat16),
                        lambda: ops.triattn_pack(*params, device=z.device))
@@ -135,12 +136,13 @@ class PairSingleBlock(nn.Module):
                               lambda: ops.pair_bias_pack(*pb_params, device=z.device))
         tiles = ops.pair_bias_project(z, pb_blob, self.num_heads, eps=self.layernorm_z.eps)
         att = self.attention
+        check_inf(att)
         params = _parameters(att)
         blob = cached_blob(att, "_hip_apb_cache", cache_key(tuple(params.values()), s, torch.bfloat16),
                            lambda: ops.apb_pack(att.channel_a, att.num_heads, _cond_channels(att),
                                                 device=s.device, **params))
         ops.apb_forward(s, None, tiles, mask.reshape(B, -1), blob, att.num_heads, 0, True, B > 1,
-                        eps=att.layernorm_a.eps, residual=s, out=s)
+                        eps=norm_eps(att), residual=s, out=s)
         hip_transition(self.transition, s, residual=s, out=s)
         return z, s
 

@@ -6,12 +6,17 @@ import torch
 from torch import nn
 
 
-def compute_dtype(x: torch.Tensor) -> torch.dtype:
-    """Autocast dtype when autocast is on, else the input dtype
-    (reference: model/primitives/triangle_multiplication.py:67-70)."""
-    if torch.is_autocast_enabled(x.device.type):
-        return torch.get_autocast_dtype(x.device.type)
-    return x.dtype
+# softmax masking: the kernels give a masked key probability exactly 0 (and attend uniformly
+# when every key of a row is masked), which is what the reference's finite ``-inf * (1 - mask)``
+# term does in fp32 for any ``inf`` large enough that exp(-inf + logit) underflows
+MIN_INF = 1e4
+
+
+def check_inf(module: nn.Module) -> None:
+    inf = getattr(module, "inf", 1e9)
+    if not inf >= MIN_INF:
+        raise NotImplementedError(
+            f"The hip backend implements hard masking (inf >= {MIN_INF:g}); got inf={inf!r}")
 
 
 def cache_key(parameters, x: torch.Tensor, dtype: torch.dtype) -> tuple:

@@ -14,7 +14,7 @@ import torch
 from torch import nn
 
 from .. import ops
-from ._common import cache_key, cached_blob, check_inference
+from ._common import cache_key, cached_blob, check_inf, check_inference
 from .layers import LayerNorm, LinearNoBias
 
 
@@ -29,6 +29,7 @@ def hip_triangular_attn(module: nn.Module, x: torch.Tensor, mask: torch.Tensor |
                         starting: bool) -> torch.Tensor:
     """x [*, I, J, C] and mask [*, I, J] in the caller's (untransposed) layout."""
     check_inference(x, "triangle attention")
+    check_inf(module)
     params = _parameters(module)
     key = cache_key(params, x, torch.bfloat16)
     blob = cached_blob(module, "_hip_attention_cache", key,

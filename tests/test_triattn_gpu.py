@@ -137,3 +137,57 @@ def test_triattn_logits_far_from_zero(shift):
     x, _, pm = synthetic.pair_inputs(n, 128, 9, seed=13)
     got, want = _run(ref, hip, x, pm, torch.bfloat16)
     assert_close(got, want, f"triattn bias shift {shift}", auto_scale=True)
+
+
+def test_triattn_fully_masked_rows_with_large_varying_logits():
+    """Rows whose keys are all masked (padded query rows; the block's final mask zeroes them).
+    The reference adds a finite -1e9 to every masked logit in fp32 (triangle_attention.py:328):
+    the spacing of fp32 at 1e9 is 64, so logits below 32 in magnitude vanish in that sum and the
+    row attends uniformly, while larger ones leave a residue that is a multiple of 64 (weights
+    then differ by factors of e^64 and flip with the last bit of q.k).  The kernel attends
+    uniformly over the N keys in every fully masked row, whatever the logits: identical to the
+    reference while |q.k|, |bias| < 32, a stated deviation beyond.  Rows with a valid key follow
+    the reference at any logit size."""
+    print("case triattn fully masked rows, large varying logits", flush=True)
+    ref, hip = _modules(True, seed=21, std=0.02)
+    g = torch.Generator().manual_seed(22)
+    with torch.no_grad():
+        for w in (ref.mha.linear_q.weight, ref.mha.linear_k.weight):
+            w.copy_(0.25 * torch.randn(w.shape, generator=g))       # |q.k| reaches ~40
+        ref.linear.weight.copy_(0.5 * torch.randn(ref.linear.weight.shape, generator=g))
+        for w in (ref.mha.linear_v.weight, ref.mha.linear_o.weight, ref.mha.linear_g.weight):
+            w.copy_(0.1 * torch.randn(w.shape, generator=g))
+    hip.load_state_dict(ref.state_dict())
+    n = 70
+    x, _, _ = synthetic.pair_inputs(n, 128, 0, seed=23)
+    mask = torch.rand(1, n, n, generator=g) > 0.3
+    dead = [5, 33, 69]
+    mask[0, dead, :] = False
+    xb = x.to(torch.bfloat16)
+    with torch.no_grad():
+        got = hip(xb.to(DEV), mask.to(DEV)).float().cpu()
+        want = ref(xb.float(), mask.float())
+        xn = ref.layer_norm(xb.float())
+        q = ref.mha.linear_q(xn[0, dead]).unflatten(-1, (4, 32)) / 32 ** 0.5
+        k = ref.mha.linear_k(xn[0, dead]).unflatten(-1, (4, 32))
+        assert torch.einsum("rqhd,rkhd->rhqk", q, k).abs().max() > 32     # residues do occur
+        live = [i for i in range(n) if i not in dead]
+        # (bf16 operands at logits of this size: only the relative gate is meaningful)
+        assert_close(got[0, live], want[0, live], "rows with a valid key, large logits",
+                     max_abs=float("inf"), mean_abs=float("inf"), rel_fro=4e-2)
+        # fully masked rows: gate * mean of v over all N keys, projected
+        v_mean = ref.mha.linear_v(xn[0, dead]).mean(dim=1, keepdim=True)           # [rows, 1, 128]
+        gate = torch.sigmoid(ref.mha.linear_g(xn[0, dead]))                         # [rows, N, 128]
+        uniform = ref.mha.linear_o(gate * v_mean)
+        assert_close(got[0, dead], uniform, "fully masked rows attend uniformly", auto_scale=True)
+        # the reference itself is far from uniform here (residues of 64): the stated deviation
+        assert (want[0, dead] - uniform).abs().max() > 10 * (got[0, dead] - uniform).abs().max()
+        # ... and agrees with the kernel once the logits are below 32: scale q down
+        ref.mha.linear_q.weight.mul_(1e-3)
+        ref.linear.weight.mul_(1e-2)
+        hip.load_state_dict(ref.state_dict())
+        got2 = hip(xb.to(DEV), mask.to(DEV)).float().cpu()
+        want2 = ref(xb.float(), mask.float())
+        assert_close(got2[0, dead], want2[0, dead], "fully masked rows, |logits| < 32", auto_scale=True)
+        assert_close(want2[0, dead], uniform, "oracle is uniform there too", auto_scale=True,
+                     max_abs=1e-4, mean_abs=1e-5, rel_fro=1e-4)
