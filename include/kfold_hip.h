@@ -144,6 +144,21 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
                            void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
                            int expansion, float eps, int io_dtype, void* stream);
 
+/* The same computation for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  The library-internal scratch that kfh_transition_forward takes as `workspace`
+ * (LayerNorm-ed rows and SwiGLU hidden activations, kfh_transition_workspace_bytes()) lives
+ * in a static device array of kfh_transition_static_scratch_bytes() = 8 MiB per GPU, held until
+ * the process ends; the call allocates and frees nothing.  Requests that need more scratch
+ * fail with KFH_EINVAL (e.g. C = 384, expansion 4: up to 2184 rows).  All calls on one GPU
+ * share the array: calls that may overlap in time on one GPU (different streams or threads)
+ * race; calls on one stream are ordered.  Results are bit-identical to
+ * kfh_transition_forward. */
+size_t kfh_transition_static_scratch_bytes(void);
+int kfh_transition_forward_static(const void* x, const void* blob, const void* residual,
+                                  const uint8_t* mask, void* out, long long rows, int C, int expansion,
+                                  float eps, int io_dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------
  * Pair bias of the token-track attention, as bf16 "bias tiles": the layout the attention
  * kernel reads, [batch][head][query block of 32][key block of 32][2 KiB tile], values

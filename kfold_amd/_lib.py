@@ -40,6 +40,8 @@ SIGNATURES: dict[str, tuple] = {
     "kfh_transition_workspace_bytes": (c_size_t, [c_longlong, c_int, c_int]),
     "kfh_transition_forward": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_longlong, c_int, c_int,
                                        c_float, c_int, _P]),
+    "kfh_transition_static_scratch_bytes": (c_size_t, []),
+    "kfh_transition_forward_static": (c_int, [_P, _P, _P, _P, _P, c_longlong, c_int, c_int, c_float, c_int, _P]),
     "kfh_bias_tiles_bytes": (c_size_t, [c_int, c_int, c_int]),
     "kfh_bias_tiles_from_dense": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P]),
     "kfh_pair_bias_packed_bytes": (c_size_t, [c_int, c_int]),

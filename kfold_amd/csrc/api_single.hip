@@ -1,6 +1,7 @@
 // C ABI, single (token) track: pair bias, pair-bias attention, generic transition.
 #include "../../include/kfold_hip.h"
 
+#include <atomic>
 #include <cmath>
 
 #include "api_util.hpp"
@@ -348,9 +349,12 @@ size_t kfh_transition_workspace_bytes(long long rows, int C, int expansion) {
     return align_up((size_t)rows * C * 2) + align_up((size_t)rows * C * expansion * 2);
 }
 
-int kfh_transition_forward(const void* x, const void* blob, const void* residual, const uint8_t* mask,
-                           void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
-                           int expansion, float eps, int io_dtype, void* stream_) {
+}  // extern "C"
+
+namespace {
+int transition_forward_impl(const void* x, const void* blob, const void* residual, const uint8_t* mask,
+                            void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
+                            int expansion, float eps, int io_dtype, void* stream_) {
     if (kfh_transition_packed_bytes(C, expansion) == 0)
         return fail(KFH_EUNSUPPORTED, "transition_forward: C=%d E=%d not supported", C, expansion);
     if (rows < 0) return fail(KFH_EINVAL, "transition_forward: rows=%lld", rows);
@@ -384,6 +388,66 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
     q.out = out; q.out_dtype = io_dtype; q.ldo = C;
     KFH_TRY(launch_linear(q, stream), "linear");
     return check_launch("transition_forward");
+}
+
+// ---- static scratch of kfh_transition_forward_static ---------------------------------------
+// Device memory beyond inputs and outputs for callers that cannot allocate: the LayerNorm-ed
+// rows and the SwiGLU hidden activations of the token-track transition.  Each GPU the library
+// runs on holds its own copy of the array until the process ends.
+constexpr size_t kStaticScratchBytes = (size_t)8 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+// Device address of `scratch` on the current device, looked up once per device.  (In host code
+// the array's name is only a handle for this lookup, never a device address.)
+int static_scratch_ptr(void** ptr) {
+    constexpr int kMaxDevices = 64;
+    static std::atomic<void*> table[kMaxDevices];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(KFH_EHIP, "transition_forward_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices) return fail(KFH_EUNSUPPORTED, "transition_forward_static: device %d", dev);
+    void* p = table[dev].load(std::memory_order_acquire);
+    if (!p) {
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return fail(KFH_EHIP, "transition_forward_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        table[dev].store(p, std::memory_order_release);     // same value from every thread
+    }
+    *ptr = p;
+    return KFH_OK;
+}
+}  // namespace
+
+extern "C" {
+
+int kfh_transition_forward(const void* x, const void* blob, const void* residual, const uint8_t* mask,
+                           void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
+                           int expansion, float eps, int io_dtype, void* stream) {
+    return transition_forward_impl(x, blob, residual, mask, out, workspace, workspace_bytes, rows, C,
+                                   expansion, eps, io_dtype, stream);
+}
+
+size_t kfh_transition_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int kfh_transition_forward_static(const void* x, const void* blob, const void* residual,
+                                  const uint8_t* mask, void* out, long long rows, int C, int expansion,
+                                  float eps, int io_dtype, void* stream) {
+    if (kfh_transition_packed_bytes(C, expansion) == 0)
+        return fail(KFH_EUNSUPPORTED, "transition_forward_static: C=%d E=%d not supported", C, expansion);
+    if (rows < 0) return fail(KFH_EINVAL, "transition_forward_static: rows=%lld", rows);
+    const size_t need = kfh_transition_workspace_bytes(rows, C, expansion);
+    if (need > kStaticScratchBytes)
+        return fail(KFH_EINVAL,
+                    "transition_forward_static: rows=%lld C=%d E=%d needs %zu bytes of scratch, the static "
+                    "buffer holds %zu (use kfh_transition_forward with a workspace)",
+                    rows, C, expansion, need, kStaticScratchBytes);
+    void* ws = nullptr;
+    if (need) {                      // the fused C = 128 kernel keeps everything in registers
+        const int rc = static_scratch_ptr(&ws);
+        if (rc) return rc;
+    }
+    return transition_forward_impl(x, blob, residual, mask, out, ws, need, rows, C, expansion, eps,
+                                   io_dtype, stream);
 }
 
 }  // extern "C"
