@@ -109,7 +109,14 @@ def test_no_cpu_fallback_in_the_product_path():
     for path in (ROOT / "kfold_amd").rglob("*.py"):
         text = path.read_text()
         assert "import oracle" not in text and "from oracle" not in text, path
-    for name in ("bench.py",):
-        # the benchmark may only use the oracle for its cpu_baseline leg
-        text = (ROOT / name).read_text()
-        assert text.count("from oracle") == 1 and "def cpu_baseline" in text
+    # the benchmark may only use the oracle for its cpu_baseline leg
+    text = (ROOT / "bench.py").read_text()
+    current = ""
+    uses = 0
+    for line in text.splitlines():
+        if line.startswith("def "):
+            current = line.split("(")[0][4:]
+        if "from oracle" in line or "import oracle" in line:
+            uses += 1
+            assert current.startswith("cpu_baseline"), f"bench.py: oracle used in {current}()"
+    assert uses >= 1
