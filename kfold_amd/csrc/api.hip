@@ -39,7 +39,7 @@ int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w
         launch_pack_blocks(g_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, -kLog2e,
                            b + kTmAbOff + (2 * cb + 1) * kBlockBytes, stream);
     }
-    launch_pack_blocks(g_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE2, K_NATURAL, -kLog2e,
+    launch_pack_blocks(g_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE4, K_NATURAL, -kLog2e,
                        b + kTmGateOff, stream);
     launch_pack_blocks(p_out_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE4, K_HALF, 1.f, b + kTmOutOff,
                        stream);
@@ -56,8 +56,7 @@ size_t kfh_trimul_workspace_bytes(int N, int C) {
     const size_t np = trimul_np(N);
     const size_t planes_ab = align_up(2 * (size_t)C * np * np * 2);
     const size_t planes_y = align_up((size_t)C * np * np * 2);
-    const size_t gate = align_up((size_t)N * N * C * 2);
-    return planes_ab + planes_y + gate;
+    return planes_ab + planes_y;
 }
 
 int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, const void* residual,
@@ -89,8 +88,6 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
     char* ws = static_cast<char*>(workspace);
     uint16_t* planes_ab = reinterpret_cast<uint16_t*>(ws);
     uint16_t* planes_y = reinterpret_cast<uint16_t*>(ws + align_up(2 * (size_t)C * np * np * 2));
-    uint16_t* gate = reinterpret_cast<uint16_t*>(reinterpret_cast<char*>(planes_y) +
-                                                 align_up((size_t)C * np * np * 2));
     const char* bl = static_cast<const char*>(blob);
     for (int b = 0; b < B; ++b) {
         const size_t off = (size_t)b * N * N * C * esz;
@@ -98,12 +95,12 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
         const char* rb = residual ? static_cast<const char*>(residual) + off : nullptr;
         char* ob = static_cast<char*>(out) + off;
         if (stages & KFH_STAGE_IN)
-            launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, gate, N, np,
+            launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, N, np,
                              direction == KFH_INCOMING, eps, stream);
         if (stages & KFH_STAGE_CORE)
             launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream);
         if (stages & KFH_STAGE_OUT)
-            launch_trimul_out(planes_y, gate, bl, rb, ob, io_dtype, N, np, eps, stream);
+            launch_trimul_out(planes_y, zb, bl, rb, ob, io_dtype, N, np, eps, stream);
     }
     return check_launch("trimul_forward");
 }

@@ -19,12 +19,11 @@ void launch_copy_f32(const void* src, int wdtype, float* dst, int n, float fill,
 
 // ---- triangle multiplication (trimul.hip, contract.hip) ------------------------------------
 // Packed weight blob of one triangle-multiplication module (C = D = 128):
-//   [0, 32K)      2 steps x { g_out blocks 2s, 2s+1 }          (ROW_INTERLEAVE2)
+//   [0, 32K)      g_out, 4 blocks                               (ROW_INTERLEAVE4), output phase
 //   [32K, 160K)   8 steps x { p_in block cb, g_in block cb }   (32 channels of a|b each)
 //                 all gate weights (g_out, g_in) are pre-multiplied by -log2(e)
 //   [160K, 192K)  p_out, 4 blocks                               (ROW_INTERLEAVE4, K_HALF)
 //   [192K, +2K)   fp32: ln_in gamma, ln_in beta, ln_out gamma, ln_out beta (128 each)
-constexpr size_t kTmInOff = 0;                       // start of the 10 input-phase steps
 constexpr size_t kTmGateOff = 0;
 constexpr size_t kTmAbOff = 4 * kBlockBytes;
 constexpr size_t kTmOutOff = 20 * kBlockBytes;
@@ -36,11 +35,10 @@ inline int round_up(int x, int m) { return (x + m - 1) / m * m; }
 inline int trimul_np(int N) { return round_up(N, 128); }
 
 void launch_trimul_in(const void* z, int io_dtype, const uint8_t* mask, const char* blob,
-                      uint16_t* planes, uint16_t* gate, int N, int Np, int incoming, float eps,
-                      hipStream_t stream);
+                      uint16_t* planes, int N, int Np, int incoming, float eps, hipStream_t stream);
 void launch_contract(const uint16_t* planes_a, const uint16_t* planes_b, uint16_t* planes_y,
                      int Np, int D, hipStream_t stream);
-void launch_trimul_out(const uint16_t* planes_y, const uint16_t* gate, const char* blob,
+void launch_trimul_out(const uint16_t* planes_y, const void* z, const char* blob,
                        const void* residual, void* out, int io_dtype, int N, int Np, float eps,
                        hipStream_t stream);
 
