@@ -216,6 +216,26 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
                     int bias_per_sample, int mask_per_sample, int s_per_sample, float eps,
                     int io_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * Parcae recurrence step of the trunk: replaces the torch line
+ *   z = a * z + F.linear(self.layernorm_z(u_t), b)             (model/model.py:528)
+ * with a, b from `_parcae_discretized_dynamics` (model/model.py:272-277):
+ *   delta = softplus(parcae_log_delta), a = exp(-delta * exp(parcae_log_a)),
+ *   b = delta[:, None] * parcae_b_cont.
+ * C = 128 or 256 (the shipping pair width).  One fused pass, no workspace.
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_parcae_packed_bytes(int C);
+
+/* ln_* [C] (`layernorm_z`); log_a, log_delta [C]; b_cont [C, C] ([out, in]).  The dynamics are
+ * evaluated here, once per weight update, as the reference does once per `run_trunk` call. */
+int kfh_parcae_pack(const void* ln_w, const void* ln_b, const void* log_a, const void* log_delta,
+                    const void* b_cont, int w_dtype, int C, void* blob, void* stream);
+
+/* out[r,:] = a * z[r,:] + b LN(u[r,:]) for r < rows; z, u, out: [rows, C] (io_dtype).
+ * `out` may alias `z` (the in-place update of the pair state); it must not alias `u`. */
+int kfh_parcae_step(const void* z, const void* u, const void* blob, void* out, long long rows, int C,
+                    float eps, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -199,4 +199,74 @@ __device__ __forceinline__ void stage_ln_rows(char* tile, const void* src, const
     }
 }
 
+// ---------------------------------------------------------------------------------------
+// The same staging for a channel count C that is a multiple of 128 (C = 256: the shipping pair
+// width): row stride 2*C + 16 bytes; a row is held by 16 lanes, lane ch owning the channels
+// 128*j + 8*ch + 0..7 for j < C/128 (16-byte loads, 256 contiguous bytes per 16 lanes).
+// ---------------------------------------------------------------------------------------
+template <int C> constexpr int xs_bytes() { return 2 * C + 16; }
+
+template <int C>
+__device__ __forceinline__ bf16x8 lds_frag_c(const char* tile, int row, int ks, int half) {
+    return *reinterpret_cast<const bf16x8*>(tile + row * xs_bytes<C>() + ks * 32 + half * 16);
+}
+
+template <int IO, int ROWS, int C, class RowOff, int NTHREADS = 256>
+__device__ __forceinline__ void stage_ln_rows_c(char* tile, const void* src, const float* lnp,
+                                                float eps, int tid, RowOff row_off) {
+    constexpr int NJ = C / 128;
+    constexpr int RG = NTHREADS / 16, NIT = ROWS / RG;
+    const int r16 = tid >> 4, ch = tid & 15;
+    // rows in groups of at most 4 per thread: all loads of a group are requested before the
+    // first row is normalised
+    constexpr int GROUP = NIT < 4 ? NIT : 4;
+    static_assert(NIT % GROUP == 0, "rows per thread");
+#pragma unroll 1
+    for (int g0 = 0; g0 < NIT; g0 += GROUP) {
+        float x[GROUP][NJ][8];
+        bool valid[GROUP];
+#pragma unroll
+        for (int it = 0; it < GROUP; ++it) {
+            const long long off = row_off((g0 + it) * RG + r16);
+            valid[it] = off >= 0;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+                load8<IO>(src, (size_t)(valid[it] ? off : 0) + 128 * j + ch * 8, x[it][j]);
+        }
+#pragma unroll
+        for (int it = 0; it < GROUP; ++it) {
+            const int row = (g0 + it) * RG + r16;
+            float s = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if (!valid[it]) x[it][j][i] = 0.f;
+                    s += x[it][j][i];
+                }
+            const float mean = row16_sum(s) * (1.0f / C);
+            float q = 0.f;
+#pragma unroll
+            for (int j = 0; j < NJ; ++j)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    x[it][j][i] -= mean;
+                    q += x[it][j][i] * x[it][j][i];
+                }
+            const float rstd = __builtin_amdgcn_rsqf(row16_sum(q) * (1.0f / C) + eps);
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const float* gam = lnp + 128 * j + ch * 8;
+                const float* bet = lnp + C + 128 * j + ch * 8;
+                u32x4 o;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    o[i] = pack_bf16(x[it][j][2 * i] * rstd * gam[2 * i] + bet[2 * i],
+                                     x[it][j][2 * i + 1] * rstd * gam[2 * i + 1] + bet[2 * i + 1]);
+                *reinterpret_cast<u32x4*>(tile + row * xs_bytes<C>() + 256 * j + ch * 16) = o;
+            }
+        }
+    }
+}
+
 }  // namespace kfh

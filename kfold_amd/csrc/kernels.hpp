@@ -93,6 +93,15 @@ constexpr size_t kPbBlobBytes = kBlockBytes + 2 * kC * sizeof(float);
 void launch_pair_bias(const void* z, int io_dtype, const char* blob, uint16_t* tiles, int N, int H,
                       float eps, hipStream_t stream);
 
+// ---- Parcae recurrence step (parcae.hip), C = 128 or 256 ------------------------------------
+// blob: packed B [C/32 blocks][C/16 k-steps][64][8] bf16 (ROW_INTERLEAVE4 within groups of 128
+// output channels), fp32 LN gamma, beta [2C], fp32 a [C], then C*C fp32 of pack-time scratch
+inline size_t parcae_blob_bytes(int C) { return (size_t)C * C * 2 + 3 * (size_t)C * 4 + (size_t)C * C * 4; }
+void launch_parcae_dynamics(const void* log_a, const void* log_delta, const void* b_cont, int wdtype,
+                            float* a_out, float* b_out, int C, hipStream_t stream);
+int launch_parcae_step(const void* z, const void* u, int io_dtype, const char* blob, void* out, long long M,
+                       int C, float eps, hipStream_t stream);
+
 // ---- single-track helpers (rows.hip, linear.hip) -------------------------------------------
 int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
                      long long M, int C, int normalize, float eps, hipStream_t stream);

@@ -1,0 +1,130 @@
+// Parcae recurrence step of the trunk (reference: src/kfold/model/model.py:523-529 with the
+// discretised dynamics of :272-277):
+//     delta = softplus(log_delta);  a = exp(-delta * exp(log_a));  B = delta[:, None] * b_cont
+//     z <- a * z + B LN(u)                      (F.linear: B is [out, in]; LN = layernorm_z)
+// One pass: u rows are LayerNorm-ed into LDS, multiplied with the packed B on the matrix cores
+// and added to a * z in the store epilogue.  HBM-bound: reads z and u, writes z.
+#include "kernels.hpp"
+
+namespace kfh {
+
+// a [C] fp32 and B (fp32, row-major [C, C]) from the module's parameters
+template <int WT>
+__global__ void parcae_dynamics_kernel(const void* __restrict__ log_a, const void* __restrict__ log_delta,
+                                       const void* __restrict__ b_cont, float* __restrict__ a_out,
+                                       float* __restrict__ b_out, int C) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= C * C) return;
+    auto rd = [](const void* p, int k) -> float {
+        if constexpr (WT == KFH_F32) return static_cast<const float*>(p)[k];
+        else return bf16_lo(static_cast<const uint16_t*>(p)[k]);
+    };
+    const int r = i / C;
+    const float ld = rd(log_delta, r);
+    const float delta = ld > 20.f ? ld : log1pf(expf(ld));          // softplus, torch's threshold
+    b_out[i] = delta * rd(b_cont, i);
+    if (i % C == 0) a_out[r] = expf(-delta * expf(rd(log_a, r)));
+}
+
+// 128 positions per workgroup, 32 per wavefront; output channels in groups of 128 (4 blocks,
+// ROW_INTERLEAVE4: block nb, lane col <-> channel 128*g + 4*col + nb).
+template <int IO, int C>
+__global__ __launch_bounds__(256, 3) void parcae_step_kernel(const void* z, const void* __restrict__ u,
+                                                             const char* __restrict__ blob, void* out,
+                                                             long long M, float eps) {
+    constexpr int KS = C / 16;
+    __shared__ __attribute__((aligned(16))) char smem[128 * xs_bytes<C>()];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const long long p0 = (long long)blockIdx.x * 128;
+    const size_t w_bytes = (size_t)C * C * 2;
+    const float* lnp = reinterpret_cast<const float*>(blob + w_bytes);
+    const float* av = lnp + 2 * C;
+    auto row_off = [&](int row) -> long long {
+        const long long p = p0 + row;
+        return p < M ? p * C : -1;
+    };
+    stage_ln_rows_c<IO, 128, C, decltype(row_off), 256>(smem, u, lnp, eps, tid, row_off);
+    __syncthreads();
+    bf16x8 xf[KS];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) xf[ks] = lds_frag_c<C>(smem, 32 * wave + col, ks, half);
+    const bf16x8* w = reinterpret_cast<const bf16x8*>(blob);
+#pragma unroll 1
+    for (int g = 0; g < C / 128; ++g) {
+        f32x16 acc[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[nb][v] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                acc[nb] = mfma32(xf[ks], w[((size_t)(4 * g + nb) * KS + ks) * 64 + lane], acc[nb]);
+            __builtin_amdgcn_sched_barrier(0);      // keep the weight loads of later blocks out of flight
+        }
+        const int c0 = 128 * g + 4 * col;
+        const float a0 = av[c0], a1 = av[c0 + 1], a2 = av[c0 + 2], a3 = av[c0 + 3];
+        // rows in two groups of 8: the z values of a group are requested before its first store
+        // (out may alias z: a lane reads a row before it writes it)
+#pragma unroll
+        for (int h8 = 0; h8 < 2; ++h8) {
+            u32x2 zb[8];
+            f32x4 zf[8];
+#pragma unroll
+            for (int uu = 0; uu < 8; ++uu) {
+                long long p = p0 + 32 * wave + acc_row(8 * h8 + uu, half);
+                p = p < M ? p : M - 1;
+                if constexpr (IO == KFH_BF16)
+                    zb[uu] = *reinterpret_cast<const u32x2*>(static_cast<const uint16_t*>(z) + p * C + c0);
+                else
+                    zf[uu] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(z) + p * C + c0);
+            }
+#pragma unroll
+            for (int uu = 0; uu < 8; ++uu) {
+                const int v = 8 * h8 + uu;
+                const long long p = p0 + 32 * wave + acc_row(v, half);
+                if (p >= M) continue;
+                if constexpr (IO == KFH_BF16) {
+                    u32x2 o = {pack_bf16(a0 * bf16_lo(zb[uu][0]) + acc[0][v], a1 * bf16_hi(zb[uu][0]) + acc[1][v]),
+                               pack_bf16(a2 * bf16_lo(zb[uu][1]) + acc[2][v], a3 * bf16_hi(zb[uu][1]) + acc[3][v])};
+                    *reinterpret_cast<u32x2*>(static_cast<uint16_t*>(out) + p * C + c0) = o;
+                } else {
+                    f32x4 o = {a0 * zf[uu][0] + acc[0][v], a1 * zf[uu][1] + acc[1][v],
+                               a2 * zf[uu][2] + acc[2][v], a3 * zf[uu][3] + acc[3][v]};
+                    *reinterpret_cast<f32x4*>(static_cast<float*>(out) + p * C + c0) = o;
+                }
+            }
+        }
+    }
+}
+
+void launch_parcae_dynamics(const void* log_a, const void* log_delta, const void* b_cont, int wdtype,
+                            float* a_out, float* b_out, int C, hipStream_t stream) {
+    const int n = C * C;
+    if (wdtype == KFH_F32)
+        hipLaunchKernelGGL(parcae_dynamics_kernel<KFH_F32>, dim3((n + 255) / 256), dim3(256), 0, stream, log_a,
+                           log_delta, b_cont, a_out, b_out, C);
+    else
+        hipLaunchKernelGGL(parcae_dynamics_kernel<KFH_BF16>, dim3((n + 255) / 256), dim3(256), 0, stream, log_a,
+                           log_delta, b_cont, a_out, b_out, C);
+}
+
+int launch_parcae_step(const void* z, const void* u, int io_dtype, const char* blob, void* out, long long M,
+                       int C, float eps, hipStream_t stream) {
+    if (M <= 0) return 0;
+    if (M > 0x7fffffffLL * 128) return -1;
+    dim3 grid((unsigned)((M + 127) / 128)), block(256);
+#define KFH_PARCAE(IO, CC) \
+    hipLaunchKernelGGL((parcae_step_kernel<IO, CC>), grid, block, 0, stream, z, u, blob, out, M, eps)
+    if (C == 128) {
+        if (io_dtype == KFH_F32) KFH_PARCAE(KFH_F32, 128); else KFH_PARCAE(KFH_BF16, 128);
+    } else if (C == 256) {
+        if (io_dtype == KFH_F32) KFH_PARCAE(KFH_F32, 256); else KFH_PARCAE(KFH_BF16, 256);
+    } else {
+        return -1;
+    }
+#undef KFH_PARCAE
+    return 0;
+}
+
+}  // namespace kfh

@@ -161,3 +161,31 @@ class PairformerTrunk(nn.Module):
         for blk in self.blocks:
             z, s = blk(z, s, pair_mask, mask, inplace_output=True)
         return z, s
+
+
+class ParcaeStep(nn.Module):
+    """The trunk's Parcae recurrence ``z <- a * z + B LN(u)`` (reference:
+    src/kfold/model/model.py:523-529; parameters named as on ``KFold``, :201-217:
+    ``layernorm_z``, ``parcae_log_a``, ``parcae_log_delta``, ``parcae_b_cont``).  One fused kernel;
+    ``z`` is updated in place unless ``inplace=False``."""
+
+    def __init__(self, channel_z: int = 256, decay_init: float = 0.9, kernel_backend: str = "hip"):
+        super().__init__()
+        import math
+
+        self.kernel_backend = kernel_backend
+        self.channel_z = channel_z
+        self.layernorm_z = LayerNorm(channel_z)
+        self.parcae_log_a = nn.Parameter(torch.zeros(channel_z))
+        delta_init = -math.log(decay_init)
+        self.parcae_log_delta = nn.Parameter(torch.full((channel_z,), math.log(math.expm1(delta_init))))
+        self.parcae_b_cont = nn.Parameter(torch.eye(channel_z))
+
+    def forward(self, z: torch.Tensor, u: torch.Tensor, inplace: bool = True) -> torch.Tensor:
+        check_inference(z, "Parcae step")
+        _contiguous_io(z, "z")
+        params = (self.layernorm_z.weight, self.layernorm_z.bias, self.parcae_log_a, self.parcae_log_delta,
+                  self.parcae_b_cont)
+        blob = cached_blob(self, "_hip_parcae_cache", cache_key(params, z, torch.bfloat16),
+                           lambda: ops.parcae_pack(*params, device=z.device))
+        return ops.parcae_step(z, u.contiguous(), blob, eps=self.layernorm_z.eps, out=z if inplace else None)

@@ -312,3 +312,42 @@ def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tenso
                                 1 if sc is not None and sc.shape[0] == S and S > 1 else 0,
                                 float(eps), _io_dtype(ac), _stream(dev)))
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# Parcae recurrence step
+# ---------------------------------------------------------------------------------------
+def parcae_pack(ln_w, ln_b, log_a, log_delta, b_cont, device: torch.device) -> torch.Tensor:
+    L = _lib.lib()
+    C = b_cont.shape[0]
+    nbytes = L.kfh_parcae_packed_bytes(C)
+    if nbytes == 0:
+        raise NotImplementedError(f"hip Parcae step is built for C=128 and C=256, got {C}")
+    ws = _weights_f32(device, ln_w, ln_b, log_a, log_delta, b_cont)
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        check(L.kfh_parcae_pack(*[_ptr(w) for w in ws], KFH_F32, C, blob.data_ptr(), _stream(device)))
+    return blob
+
+
+def parcae_step(z: torch.Tensor, u: torch.Tensor, blob: torch.Tensor, eps: float = 1e-5,
+                out: torch.Tensor | None = None) -> torch.Tensor:
+    """``out = a * z + b LN(u)`` over the last dim; ``out`` may be ``z`` (in place)."""
+    dev = _require_cuda(z, u, blob, out)
+    if u.shape != z.shape or u.dtype != z.dtype:
+        raise ValueError("z and u must have the same shape and dtype")
+    C = z.shape[-1]
+    rows = z.numel() // C if z.numel() else 0
+    if not z.is_contiguous() or not u.is_contiguous():
+        raise ValueError("z and u must be contiguous")
+    if out is None:
+        out = torch.empty_like(z)
+    elif out.shape != z.shape or out.dtype != z.dtype or not out.is_contiguous():
+        raise ValueError("out must be contiguous with the shape and dtype of z")
+    if rows == 0:
+        return out
+    L = _lib.lib()
+    with torch.cuda.device(dev):
+        check(L.kfh_parcae_step(z.data_ptr(), u.data_ptr(), blob.data_ptr(), out.data_ptr(), rows, C,
+                                float(eps), _io_dtype(z), _stream(dev)))
+    return out

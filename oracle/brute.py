@@ -164,3 +164,20 @@ def adaln(a, s, p):
         bs = _lin(sn, p["linear_bias.weight"])
         out[r] = [_sig(gt[c]) * an[c] + bs[c] for c in range(len(an))]
     return out
+
+
+def parcae_step(z, u, p):
+    """model.py:272-277 and :528.  z, u [R, C]; p: layernorm_z.{weight,bias}, parcae_log_a,
+    parcae_log_delta [C], parcae_b_cont [C, C] (row = output channel)."""
+    R, C = z.shape
+    delta = [math.log1p(math.exp(t)) for t in p["parcae_log_delta"]]
+    a = [math.exp(-delta[c] * math.exp(p["parcae_log_a"][c])) for c in range(C)]
+    out = np.zeros((R, C))
+    for r in range(R):
+        un = _ln(u[r], p["layernorm_z.weight"], p["layernorm_z.bias"])
+        for o in range(C):
+            acc = 0.0
+            for c in range(C):
+                acc += delta[o] * p["parcae_b_cont"][o][c] * un[c]
+            out[r, o] = a[o] * z[r, o] + acc
+    return out

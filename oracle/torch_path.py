@@ -424,3 +424,30 @@ class PairformerTrunk(nn.Module):
         for blk in self.blocks:
             z, s = blk(z, s, pair_mask, mask)
         return z, s
+
+
+# ---------------------------------------------------------------------------
+# Parcae recurrence of the trunk
+# ---------------------------------------------------------------------------
+class ParcaeStep(nn.Module):
+    """model/model.py:201-217 (parameters), :272-277 (discretised dynamics), :523-529 (the step
+    ``z = a * z + F.linear(layernorm_z(u), b)``).  fp32 throughout (the reference casts ``a`` and
+    ``b`` to its autocast dtype, :505)."""
+
+    def __init__(self, channel_z: int = 256, decay_init: float = 0.9):
+        super().__init__()
+        self.layernorm_z = LayerNorm(channel_z)
+        self.parcae_log_a = nn.Parameter(torch.zeros(channel_z))
+        delta_init = -math.log(decay_init)
+        self.parcae_log_delta = nn.Parameter(torch.full((channel_z,), math.log(math.expm1(delta_init))))
+        self.parcae_b_cont = nn.Parameter(torch.eye(channel_z))
+
+    def dynamics(self):
+        delta = F.softplus(self.parcae_log_delta)                    # :274
+        a = torch.exp(-delta * torch.exp(self.parcae_log_a))         # :275
+        b = delta[:, None] * self.parcae_b_cont                      # :276
+        return a, b
+
+    def forward(self, z: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+        a, b = self.dynamics()
+        return a * z + F.linear(self.layernorm_z(u), b)              # :528

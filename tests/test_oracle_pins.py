@@ -235,3 +235,33 @@ def test_block_wiring_and_in_place_residuals():
     assert torch.allclose(z_out, zz, atol=1e-10) and torch.allclose(s_out, ss, atol=1e-10)
     # eval-mode adds mutate the caller's tensors (the final mask multiply does not)
     assert not torch.equal(z_in, z) and torch.equal(s_in, s_out)
+
+
+# ------------------------------------------------------------------------ Parcae recurrence
+def test_parcae_step_vs_brute_and_closed_forms():
+    m = O.ParcaeStep(6)
+    g = torch.Generator().manual_seed(31)
+    with torch.no_grad():
+        m.parcae_log_a.copy_(0.5 * torch.randn(6, generator=g))
+        m.parcae_log_delta.copy_(torch.randn(6, generator=g))
+        m.parcae_b_cont.copy_(torch.randn(6, 6, generator=g))          # not symmetric: [out, in] matters
+        m.layernorm_z.weight.copy_(1 + 0.3 * torch.randn(6, generator=g))
+        m.layernorm_z.bias.copy_(0.3 * torch.randn(6, generator=g))
+    m = m.double().eval()
+    z, u = _rand((5, 6), 32), _rand((5, 6), 33)
+    got = m(z, u).detach().numpy()
+    want = brute.parcae_step(z.numpy(), u.numpy(), _np_params(m))
+    assert np.allclose(got, want, atol=1e-10)
+    # freshly constructed module: a = decay_init exactly, B = -log(decay_init) * I
+    f = O.ParcaeStep(4, decay_init=0.8).double()
+    a, b = f.dynamics()
+    assert torch.allclose(a, torch.full((4,), 0.8, dtype=torch.float64), atol=1e-12)
+    assert torch.allclose(b, -math.log(0.8) * torch.eye(4, dtype=torch.float64), atol=1e-12)
+    # b_cont = 0: pure channel-wise decay; log_delta -> -inf side: delta -> 0, a -> 1, state kept
+    with torch.no_grad():
+        f.parcae_b_cont.zero_()
+    zz, uu = _rand((3, 4), 34), _rand((3, 4), 35)
+    assert torch.allclose(f(zz, uu), 0.8 * zz, atol=1e-12)
+    with torch.no_grad():
+        f.parcae_log_delta.fill_(-40.0)
+    assert torch.allclose(f(zz, uu), zz, atol=1e-12)
