@@ -20,18 +20,45 @@ const char* kfh_last_error(void) { return kfh::g_err; }
 // ------------------------------------------------------------------------------------------
 // triangle multiplication
 // ------------------------------------------------------------------------------------------
-size_t kfh_trimul_packed_bytes(int C) { return C == kC ? align_up(kTmBlobBytes) : 0; }
+namespace {
+bool trimul_wide(int C) { return C == 256; }
+}  // namespace
+
+size_t kfh_trimul_packed_bytes(int C) {
+    if (trimul_wide(C)) return align_up(trimul_wide_blob_bytes(C));
+    return C == kC ? align_up(kTmBlobBytes) : 0;
+}
 
 int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w,
                     const void* g_in_w, const void* ln_out_w, const void* ln_out_b,
                     const void* p_out_w, const void* g_out_w, int w_dtype, int C, void* blob,
                     void* stream_) {
-    if (C != kC) return fail(KFH_EUNSUPPORTED, "trimul_pack: C=%d, only C=128 is built", C);
+    if (C != kC && !trimul_wide(C))
+        return fail(KFH_EUNSUPPORTED, "trimul_pack: C=%d, built for C=128 and C=256", C);
     if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "trimul_pack: bad w_dtype %d", w_dtype);
     if (!p_in_w || !g_in_w || !p_out_w || !g_out_w || !blob)
         return fail(KFH_EINVAL, "trimul_pack: null weight or blob pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     char* b = static_cast<char*>(blob);
+    if (trimul_wide(C)) {
+        size_t o_gate, o_ab, o_out, o_ln, blk;
+        trimul_wide_offsets(C, &o_gate, &o_ab, &o_out, &o_ln, &blk);
+        for (int cb = 0; cb < 2 * C / 32; ++cb) {
+            launch_pack_blocks(p_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, 1.f,
+                               b + o_ab + (2 * cb) * blk, stream);
+            launch_pack_blocks(g_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, -kLog2e,
+                               b + o_ab + (2 * cb + 1) * blk, stream);
+        }
+        launch_pack_blocks(g_out_w, w_dtype, C, C, C, 0, C / 32, ROW_INTERLEAVE4, K_NATURAL, -kLog2e, b + o_gate,
+                           stream);
+        launch_pack_blocks(p_out_w, w_dtype, C, C, C, 0, C / 32, ROW_INTERLEAVE4, K_HALF, 1.f, b + o_out, stream);
+        float* lnw = reinterpret_cast<float*>(b + o_ln);
+        launch_copy_f32(ln_in_w, w_dtype, lnw, C, 1.f, stream);
+        launch_copy_f32(ln_in_b, w_dtype, lnw + C, C, 0.f, stream);
+        launch_copy_f32(ln_out_w, w_dtype, lnw + 2 * C, C, 1.f, stream);
+        launch_copy_f32(ln_out_b, w_dtype, lnw + 3 * C, C, 0.f, stream);
+        return check_launch("trimul_pack");
+    }
     // input phase: step cb = { p_in rows 32cb.., g_in rows 32cb.. }
     for (int cb = 0; cb < 8; ++cb) {
         launch_pack_blocks(p_in_w, w_dtype, 32, C, C, 32 * cb, 1, ROW_NATURAL, K_NATURAL, 1.f,
@@ -52,7 +79,7 @@ int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w
 }
 
 size_t kfh_trimul_workspace_bytes(int N, int C) {
-    if (C != kC || N <= 0) return 0;
+    if ((C != kC && !trimul_wide(C)) || N <= 0) return 0;
     const size_t np = trimul_np(N);
     const size_t planes_ab = align_up(2 * (size_t)C * np * np * 2);
     const size_t planes_y = align_up((size_t)C * np * np * 2);
@@ -70,7 +97,8 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
                               const void* residual, void* out, void* workspace,
                               size_t workspace_bytes, int B, int N, int C, int direction, float eps,
                               int io_dtype, int stages, void* stream_) {
-    if (C != kC) return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d, only C=128 is built", C);
+    if (C != kC && !trimul_wide(C))
+        return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d, built for C=128 and C=256", C);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "trimul_forward: bad shape B=%d N=%d", B, N);
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "trimul_forward: bad io_dtype %d", io_dtype);
     if (direction != KFH_OUTGOING && direction != KFH_INCOMING)
@@ -94,13 +122,22 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
         const char* zb = static_cast<const char*>(z) + off;
         const char* rb = residual ? static_cast<const char*>(residual) + off : nullptr;
         char* ob = static_cast<char*>(out) + off;
-        if (stages & KFH_STAGE_IN)
-            launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, N, np,
-                             direction == KFH_INCOMING, eps, stream);
+        if (stages & KFH_STAGE_IN) {
+            if (trimul_wide(C))
+                launch_trimul_in_wide(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, N, np, C,
+                                      direction == KFH_INCOMING, eps, stream);
+            else
+                launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, N, np,
+                                 direction == KFH_INCOMING, eps, stream);
+        }
         if (stages & KFH_STAGE_CORE)
             launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream);
-        if (stages & KFH_STAGE_OUT)
-            launch_trimul_out(planes_y, zb, bl, rb, ob, io_dtype, N, np, eps, stream);
+        if (stages & KFH_STAGE_OUT) {
+            if (trimul_wide(C))
+                launch_trimul_out_wide(planes_y, zb, bl, rb, ob, io_dtype, N, np, C, eps, stream);
+            else
+                launch_trimul_out(planes_y, zb, bl, rb, ob, io_dtype, N, np, eps, stream);
+        }
     }
     return check_launch("trimul_forward");
 }

@@ -42,6 +42,14 @@ void launch_trimul_out(const uint16_t* planes_y, const void* z, const char* blob
                        const void* residual, void* out, int io_dtype, int N, int Np, float eps,
                        hipStream_t stream);
 
+// other pair widths (trimul_wide.hip; C = 256): same interface, blob layout in that file
+size_t trimul_wide_blob_bytes(int C);
+void trimul_wide_offsets(int C, size_t* gate, size_t* ab, size_t* out, size_t* ln, size_t* blk);
+int launch_trimul_in_wide(const void* z, int io_dtype, const uint8_t* mask, const char* blob, uint16_t* planes,
+                          int N, int Np, int C, int incoming, float eps, hipStream_t stream);
+int launch_trimul_out_wide(const uint16_t* planes_y, const void* z, const char* blob, const void* residual,
+                           void* out, int io_dtype, int N, int Np, int C, float eps, hipStream_t stream);
+
 // ---- triangle attention (triattn.hip) ------------------------------------------------------
 // Packed weight blob of one triangle-attention module (C = 128, 4 heads x 32):
 //   [0, 144K)     9 steps x 2 blocks: {q_h,k_h} h=0..3, {g_h,v_h} h=0..3, {pair bias, zero};

@@ -1,0 +1,80 @@
+"""The pair widths the shipping model uses (configs/kfold.yaml of the reference): triangle
+multiplication and the trunk's TriangularBlock at c_z = 256 (model/modules/tri_stack.py:119-125)."""
+
+import pytest
+import torch
+
+from kfold_amd import synthetic
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def _affine(ref, seed=77):
+    g = torch.Generator().manual_seed(seed)
+    with torch.no_grad():
+        for name, p in ref.named_parameters():
+            if p.dim() == 1:
+                if name.endswith("bias"):
+                    p.copy_(0.1 * torch.randn(p.shape, generator=g))
+                else:
+                    p.copy_(1 + 0.2 * torch.randn(p.shape, generator=g))
+
+
+@pytest.mark.parametrize("direction", ["outgoing", "incoming"])
+@pytest.mark.parametrize("n,n_pad,dtype", [(70, 9, torch.bfloat16), (130, 0, torch.bfloat16), (33, 4, torch.float32)])
+def test_trimul_c256(direction, n, n_pad, dtype):
+    from kfold_amd import ops, primitives as P
+    from oracle import torch_path as O
+
+    print(f"case trimul C=256 {direction} n={n} {dtype}", flush=True)
+    cls = "TriangleMultiplicationOutgoing" if direction == "outgoing" else "TriangleMultiplicationIncoming"
+    ref = getattr(O, cls)(256).eval()
+    synthetic.init_weights_(ref, 3)
+    _affine(ref)
+    hip = getattr(P, cls)(256).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    z, _, pm = synthetic.pair_inputs(n, 256, n_pad, seed=n)
+    if n == 130:        # a general (not outer-product) mask
+        pm = torch.rand(1, n, n, generator=torch.Generator().manual_seed(5)) > 0.3
+    zi = z.to(dtype)
+    with torch.no_grad():
+        want = ref(zi.float(), pm)
+        zd, pmd = zi.to(DEV), pm.to(DEV)
+        got = hip(zd, pmd)
+        assert got.dtype == dtype
+        print(assert_close(got, want, f"trimul C=256 {direction}"), flush=True)
+        assert torch.equal(got, hip(zd, pmd)), "run-to-run results differ"
+        # fused residual in place
+        zin = zd.clone()
+        ops.trimul_forward(zin, pmd, hip._hip_multiplication_cache, direction, residual=zin, out=zin)
+        assert_close(zin, zi.float() + want, "trimul C=256 residual in place", rel_fro=5e-3)
+
+
+def test_triangular_block_c256():
+    """The shipping trunk block: tri-mul out, tri-mul in, transition x4 at c_z = 256, in place."""
+    from kfold_amd import modules as M
+    from oracle import torch_path as O
+
+    print("case triangular block C=256", flush=True)
+    ref = O.TriangularBlock(256).eval()
+    synthetic.init_weights_(ref, 11)
+    hip = M.TriangularBlock(256).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    n = 80
+    z, _, pm = synthetic.pair_inputs(n, 256, 10, seed=12)
+    zb = z.bfloat16()
+    with torch.no_grad():
+        zw = ref(zb.float(), pm.float())
+        zin = zb.float().to(DEV)
+        zg = hip(zin, pm.to(DEV))
+        assert zg.data_ptr() == zin.data_ptr()
+        print(assert_close(zg, zw, "triangular block C=256 (fp32 stream)", rel_fro=5e-3), flush=True)
+        zg16 = hip(zb.to(DEV), pm.to(DEV))
+        # bf16 stream: three storage roundings of |z| up to ~5 on top of the kernel error
+        print(assert_close(zg16, zw, "triangular block C=256 (bf16 stream)", max_abs=6e-2, mean_abs=4e-3,
+                           rel_fro=5e-3), flush=True)
