@@ -158,19 +158,28 @@ TaSizes ta_sizes(int N) {
 }
 }  // namespace
 
+namespace {
+bool triattn_fused(int C, int H) { return C == kC && H == 4; }
+}  // namespace
+
 size_t kfh_triattn_packed_bytes(int C, int H) {
-    return (C == kC && H == 4) ? align_up(kTaBlobBytes) : 0;
+    return triattn_fused(C, H) ? align_up(kTaBlobBytes) : triattn_generic_blob_bytes(C, H);
 }
 
 int kfh_triattn_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* k_w,
                      const void* v_w, const void* g_w, const void* bias_w, const void* o_w,
                      int w_dtype, int C, int H, void* blob, void* stream_) {
-    if (C != kC || H != 4)
-        return fail(KFH_EUNSUPPORTED, "triattn_pack: C=%d H=%d, only C=128 H=4 is built", C, H);
+    if (!triattn_fused(C, H) && triattn_generic_blob_bytes(C, H) == 0)
+        return fail(KFH_EUNSUPPORTED, "triattn_pack: C=%d H=%d (C a multiple of 32, head dim <= 64)", C, H);
     if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "triattn_pack: bad w_dtype %d", w_dtype);
     if (!q_w || !k_w || !v_w || !g_w || !bias_w || !o_w || !blob)
         return fail(KFH_EINVAL, "triattn_pack: null weight or blob pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (!triattn_fused(C, H)) {
+        if (triattn_generic_pack(ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w, w_dtype, C, H, blob, stream))
+            return fail(KFH_EUNSUPPORTED, "triattn_pack: C=%d H=%d not built", C, H);
+        return check_launch("triattn_pack");
+    }
     char* b = static_cast<char*>(blob);
     const float qscale = kLog2e / sqrtf((float)(C / H));
     for (int h = 0; h < 4; ++h) {
@@ -194,7 +203,8 @@ int kfh_triattn_pack(const void* ln_w, const void* ln_b, const void* q_w, const 
 }
 
 size_t kfh_triattn_workspace_bytes(int N, int C, int H) {
-    if (C != kC || H != 4 || N <= 0 || N > 8192) return 0;
+    if (N <= 0 || N > 8192) return 0;
+    if (!triattn_fused(C, H)) return triattn_generic_ws_bytes(N, C, H);
     return ta_sizes(N).total;
 }
 
@@ -209,8 +219,8 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
                                const void* residual, void* out, void* workspace,
                                size_t workspace_bytes, int B, int N, int C, int H, int ending,
                                float eps, int io_dtype, int stages, void* stream_) {
-    if (C != kC || H != 4)
-        return fail(KFH_EUNSUPPORTED, "triattn_forward: C=%d H=%d, only C=128 H=4 is built", C, H);
+    if (!triattn_fused(C, H) && triattn_generic_blob_bytes(C, H) == 0)
+        return fail(KFH_EUNSUPPORTED, "triattn_forward: C=%d H=%d (C a multiple of 32, head dim <= 64)", C, H);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "triattn_forward: bad shape B=%d N=%d", B, N);
     if (N > 8192) return fail(KFH_EUNSUPPORTED, "triattn_forward: N=%d > 8192", N);
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "triattn_forward: bad io_dtype %d", io_dtype);
@@ -218,10 +228,25 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
         return fail(KFH_EINVAL, "triattn_forward: null pointer argument");
     if (out == x && residual != x)
         return fail(KFH_EINVAL, "triattn_forward: out may alias x only when residual == x");
+    hipStream_t stream = static_cast<hipStream_t>(stream_);
+    if (!triattn_fused(C, H)) {
+        const size_t need = triattn_generic_ws_bytes(N, C, H);
+        if (workspace_bytes < need)
+            return fail(KFH_EINVAL, "triattn_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+        const size_t esz_g = io_dtype == KFH_F32 ? 4 : 2;
+        for (int b = 0; b < B; ++b) {       // batch elements (templates) in turn through one workspace
+            const size_t off = (size_t)b * N * N * C * esz_g;
+            const int rc = triattn_generic_forward(
+                static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N, static_cast<const char*>(blob),
+                static_cast<char*>(workspace), residual ? static_cast<const char*>(residual) + off : nullptr,
+                static_cast<char*>(out) + off, N, C, H, ending, eps, stages, stream);
+            if (rc) return fail(KFH_EUNSUPPORTED, "triattn_forward: shape not built (%d)", rc);
+        }
+        return check_launch("triattn_forward");
+    }
     const TaSizes sz = ta_sizes(N);
     if (workspace_bytes < sz.total)
         return fail(KFH_EINVAL, "triattn_forward: workspace %zu < %zu bytes", workspace_bytes, sz.total);
-    hipStream_t stream = static_cast<hipStream_t>(stream_);
     char* w = static_cast<char*>(workspace);
     TriattnWorkspace ws;
     ws.qf = w; ws.kf = w + sz.frag; ws.vf = w + 2 * sz.frag; ws.gf = w + 3 * sz.frag;

@@ -86,6 +86,16 @@ int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char*
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
                     float eps, int stages, hipStream_t stream);
 
+// other widths / head shapes (triattn_generic.hip): head dim <= 64, C a multiple of 32
+size_t triattn_generic_blob_bytes(int C, int H);
+size_t triattn_generic_ws_bytes(int N, int C, int H);
+int triattn_generic_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* k_w, const void* v_w,
+                         const void* g_w, const void* bias_w, const void* o_w, int w_dtype, int C, int H,
+                         void* blob, hipStream_t stream);
+int triattn_generic_forward(const void* x, int io_dtype, const uint8_t* mask, const char* blob, char* ws,
+                            const void* residual, void* out, int N, int C, int H, int ending, float eps,
+                            int stages, hipStream_t stream);
+
 // ---- pair transition (transition.hip) ----------------------------------------------------
 // Packed blob (C = 128, expansion E): 4E steps x 24 KiB { u block, v block, W_out slice of the
 // step's 32 hidden channels as 4 blocks x 2 k-steps (ROW_INTERLEAVE4, K_ACC) }, then fp32 LN
@@ -111,12 +121,15 @@ int launch_parcae_step(const void* z, const void* u, int io_dtype, const char* b
                        int C, float eps, hipStream_t stream);
 
 // ---- single-track helpers (rows.hip, linear.hip) -------------------------------------------
+// transpose_n > 0: the M = n*n rows are written transposed as an [n, n] grid of rows
 int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
-                     long long M, int C, int normalize, float eps, hipStream_t stream);
+                     long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n = 0);
+// mask element of (row a, key k) is mask[a * mask_stride + k * key_stride]
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
-                      long long mask_stride, hipStream_t stream);
+                      long long mask_stride, hipStream_t stream, long long key_stride = 1);
+// source element (t = batch*H + head, q, k) at t*st + q*sq + k*sk; all zero = dense [.., H, L, L]
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
-                       hipStream_t stream);
+                       hipStream_t stream, long long st = 0, long long sq = 0, long long sk = 0);
 
 enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS };
 
@@ -133,6 +146,7 @@ struct LinearArgs {
     void* out; int out_dtype; long long ldo; int Nout;
     int epi;
     int H, PB, Dh;                               // heads, 32-blocks per padded head, real head dim
+    int out_transposed;                          // EPI_RESID: out / aux row of (a, position) is position * rows_a + a
 };
 int launch_linear(const LinearArgs& p, hipStream_t stream);
 

@@ -131,8 +131,11 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
         for (int v = 0; v < 16; ++v) {
             const int ps = blk * 32 + acc_row(v, half);
             if (ps >= p.L) continue;
-            const size_t r = (size_t)a * p.L + ps;
-            const size_t r_aux = (size_t)(p.aux_shared ? 0 : a) * p.L + ps;
+            size_t r = (size_t)a * p.L + ps;
+            size_t r_aux = (size_t)(p.aux_shared ? 0 : a) * p.L + ps;
+            if constexpr (EPI == EPI_RESID) {
+                if (p.out_transposed) { r = (size_t)ps * p.rows_a + a; r_aux = r; }
+            }
             const size_t r_gate = (size_t)(p.gate_shared ? 0 : a) * p.L + ps;
             float y = acc[v] + bc;
             if constexpr (EPI == EPI_SIGMOID) y = sigmoidf_fast(y);

@@ -11,31 +11,37 @@ __device__ __forceinline__ float wave_sum(float v) {
     return v;
 }
 
-// out[r, :] = bf16( normalize ? LN(x[r, :]) * gamma + beta : x[r, :] ), one wavefront per row.
-// gamma / beta may be null (1 / 0).  C is a multiple of 128, at most 2048.
+// out[r', :] = bf16( normalize ? LN(x[r, :]) * gamma + beta : x[r, :] ), one wavefront per row.
+// gamma / beta may be null (1 / 0).  C is even, at most 2048.  With tn > 0 the rows are the
+// positions (i, j) of a [tn, tn] grid and are written transposed: r = i * tn + j -> r' = j * tn + i.
 // (reference: model/primitives/normalization.py:61-91 — fp32 statistics, biased variance)
 template <int IO>
 __global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__ x,
                                                         const float* __restrict__ gamma,
                                                         const float* __restrict__ beta,
                                                         uint16_t* __restrict__ out, long long M, int C,
-                                                        int normalize, float eps) {
+                                                        int normalize, float eps, int tn) {
     const int lane = threadIdx.x & 63;
     const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (r >= M) return;
-    const int npair = C / 128;
+    const long long ro = tn > 0 ? (r % tn) * tn + r / tn : r;
+    const int npair = (C + 127) / 128;
     float a[16], b[16];
     float s = 0.f;
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
         if (i >= npair) break;
-        const size_t e = (size_t)r * C + 128 * i + 2 * lane;
-        if constexpr (IO == KFH_BF16) {
-            const uint32_t w = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(x) + e);
-            a[i] = bf16_lo(w); b[i] = bf16_hi(w);
-        } else {
-            const f32x2 w = *reinterpret_cast<const f32x2*>(static_cast<const float*>(x) + e);
-            a[i] = w[0]; b[i] = w[1];
+        const int c = 128 * i + 2 * lane;
+        a[i] = 0.f; b[i] = 0.f;
+        if (c < C) {
+            const size_t e = (size_t)r * C + c;
+            if constexpr (IO == KFH_BF16) {
+                const uint32_t w = *reinterpret_cast<const uint32_t*>(static_cast<const uint16_t*>(x) + e);
+                a[i] = bf16_lo(w); b[i] = bf16_hi(w);
+            } else {
+                const f32x2 w = *reinterpret_cast<const f32x2*>(static_cast<const float*>(x) + e);
+                a[i] = w[0]; b[i] = w[1];
+            }
         }
         s += a[i] + b[i];
     }
@@ -46,7 +52,7 @@ __global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             if (i >= npair) break;
-            a[i] -= mean; b[i] -= mean; q += a[i] * a[i] + b[i] * b[i];
+            if (128 * i + 2 * lane < C) { a[i] -= mean; b[i] -= mean; q += a[i] * a[i] + b[i] * b[i]; }
         }
         rstd = __builtin_amdgcn_rsqf(wave_sum(q) / C + eps);
     }
@@ -54,49 +60,53 @@ __global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__
     for (int i = 0; i < 16; ++i) {
         if (i >= npair) break;
         const int c = 128 * i + 2 * lane;
+        if (c >= C) continue;
         float u = a[i] * rstd, v = b[i] * rstd;
         if (normalize) {
             if (gamma) { u *= gamma[c]; v *= gamma[c + 1]; }
             if (beta) { u += beta[c]; v += beta[c + 1]; }
         }
-        *reinterpret_cast<uint32_t*>(out + (size_t)r * C + c) = pack_bf16(u, v);
+        *reinterpret_cast<uint32_t*>(out + (size_t)ro * C + c) = pack_bf16(u, v);
     }
 }
 
 int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
-                     long long M, int C, int normalize, float eps, hipStream_t stream) {
-    if (C % 128 || C > 2048) return -1;
+                     long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n) {
+    if (C % 2 || C > 2048 || C <= 0) return -1;
+    if (transpose_n > 0 && (long long)transpose_n * transpose_n != M) return -1;
     dim3 grid((unsigned)((M + 3) / 4)), block(256);
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(rows_norm_kernel<KFH_F32>, grid, block, 0, stream, x, gamma, beta, out, M, C,
-                           normalize, eps);
+                           normalize, eps, transpose_n);
     else
         hipLaunchKernelGGL(rows_norm_kernel<KFH_BF16>, grid, block, 0, stream, x, gamma, beta, out, M, C,
-                           normalize, eps);
+                           normalize, eps, transpose_n);
     return 0;
 }
 
-// codes[a][k] = k < L ? (mask[a * mask_stride + k] ? 2 : 1) : 0     for k < Lp = nb * 32
+// codes[a][k] = k < L ? (mask[a * row_stride + k * key_stride] ? 2 : 1) : 0     for k < Lp = nb * 32
 __global__ void key_codes_kernel(const uint8_t* __restrict__ mask, uint8_t* __restrict__ codes,
-                                 int rows, int L, int Lp, long long mask_stride) {
+                                 int rows, int L, int Lp, long long row_stride, long long key_stride) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (long long)rows * Lp) return;
     const int a = (int)(i / Lp), k = (int)(i % Lp);
-    codes[i] = k < L ? (mask[a * mask_stride + k] ? 2 : 1) : 0;
+    codes[i] = k < L ? (mask[a * row_stride + k * key_stride] ? 2 : 1) : 0;
 }
 
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
-                      long long mask_stride, hipStream_t stream) {
+                      long long mask_stride, hipStream_t stream, long long key_stride) {
     const long long n = (long long)rows * Lp;
     hipLaunchKernelGGL(key_codes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, mask,
-                       codes, rows, L, Lp, mask_stride);
+                       codes, rows, L, Lp, mask_stride, key_stride);
 }
 
 // Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled bf16 tiles (bias_tile_elem layout);
 // one thread writes the 8 keys of one (tile, chunk, lane) slot.
+// element (t, q, k) of the source is at t * st + q * sq + k * sk (t = batch * H + head)
 template <int IO>
 __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __restrict__ tiles,
-                                  long long total, int H, int L, int nb) {
+                                  long long total, int H, int L, int nb, long long st, long long sq,
+                                  long long sk) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;      // 16-byte slot
     if (i >= total) return;
     const int lane = (int)(i & 63), c = (int)((i >> 6) & 1);
@@ -113,7 +123,7 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
             const int k = kb * 32 + acc_row(8 * c + e + u, lane >> 5);
             float x = 0.f;
             if (q < L && k < L) {
-                const size_t off = ((size_t)t * L + q) * L + k;
+                const size_t off = (size_t)(t * st + q * sq + k * sk);
                 if constexpr (IO == KFH_F32) x = static_cast<const float*>(dense)[off];
                 else x = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
             }
@@ -125,13 +135,16 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
 }
 
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
-                       hipStream_t stream) {
+                       hipStream_t stream, long long st, long long sq, long long sk) {
+    if (st == 0 && sq == 0 && sk == 0) { st = (long long)L * L; sq = L; sk = 1; }    // dense [.., H, L, L]
     const long long total = (long long)nbatch * H * nb * nb * 128;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, H, L, nb);
+        hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, H, L, nb,
+                           st, sq, sk);
     else
-        hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, H, L, nb);
+        hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, H, L, nb,
+                           st, sq, sk);
 }
 
 }  // namespace kfh

@@ -32,7 +32,9 @@ def test_size_queries_and_argument_errors_need_no_gpu():
 
     lib = _lib.lib()
     assert lib.kfh_trimul_packed_bytes(128) > 0 and lib.kfh_trimul_packed_bytes(64) == 0
-    assert lib.kfh_triattn_packed_bytes(128, 4) > 0 and lib.kfh_triattn_packed_bytes(128, 8) == 0
+    assert lib.kfh_trimul_packed_bytes(256) > lib.kfh_trimul_packed_bytes(128)
+    assert lib.kfh_triattn_packed_bytes(128, 4) > 0 and lib.kfh_triattn_packed_bytes(128, 3) == 0
+    assert lib.kfh_triattn_packed_bytes(64, 4) > 0 and lib.kfh_triattn_packed_bytes(128, 1) == 0   # head dim > 64
     # workspace grows with N and is 256-byte granular
     w1, w2 = lib.kfh_trimul_workspace_bytes(384, 128), lib.kfh_trimul_workspace_bytes(768, 128)
     assert 0 < w1 < w2 and w1 % 256 == 0

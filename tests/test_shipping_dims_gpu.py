@@ -1,5 +1,7 @@
 """The pair widths the shipping model uses (configs/kfold.yaml of the reference): triangle
-multiplication and the trunk's TriangularBlock at c_z = 256 (model/modules/tri_stack.py:119-125)."""
+multiplication and the trunk's TriangularBlock at c_z = 256 (model/modules/tri_stack.py:119-125),
+triangle attention at c = 64 with 4 heads of 16 batched over templates
+(model/modules/apo_module.py:376-384)."""
 
 import pytest
 import torch
@@ -78,3 +80,42 @@ def test_triangular_block_c256():
         # bf16 stream: three storage roundings of |z| up to ~5 on top of the kernel error
         print(assert_close(zg16, zw, "triangular block C=256 (bf16 stream)", max_abs=6e-2, mean_abs=4e-3,
                            rel_fro=5e-3), flush=True)
+
+
+@pytest.mark.parametrize("starting", [True, False])
+@pytest.mark.parametrize("c,h,n,batch", [(64, 4, 50, 4), (64, 4, 128, 1), (96, 2, 37, 2)])
+def test_triattn_other_widths_batched(starting, c, h, n, batch):
+    """c = 64, 4 heads x 16 with a leading batch of 4 (the apo stack's shape); 2 heads x 48 covers
+    the 64-wide padded head."""
+    from kfold_amd import ops, primitives as P
+    from oracle import torch_path as O
+
+    print(f"case triattn c={c} h={h} n={n} batch={batch} starting={starting}", flush=True)
+    cls = "TriangleAttentionStartingNode" if starting else "TriangleAttentionEndingNode"
+    ref = getattr(O, cls)(c, h).eval()
+    synthetic.init_weights_(ref, 13, std=0.08)
+    _affine(ref)
+    hip = getattr(P, cls)(c, h).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(batch, n, n, c, generator=g).bfloat16()
+    mask = torch.rand(batch, n, n, generator=g) > 0.25
+    mask[0, 3, :] = False                 # a fully masked row / column
+    mask[0, :, 5] = False
+    if batch > 1:
+        mask[1] = synthetic.pair_mask_from_tokens(synthetic.token_mask(n, 7))[0]
+    with torch.no_grad():
+        want = torch.stack([ref(x[b:b + 1].float(), mask[b:b + 1].float())[0] for b in range(batch)])
+        xd, md = x.to(DEV), mask.to(DEV)
+        got = hip(xd, md)
+        assert got.shape == x.shape and got.dtype == x.dtype
+        print(assert_close(got, want, f"triattn c={c} h={h}", auto_scale=True), flush=True)
+        assert torch.equal(got, hip(xd, md)), "run-to-run results differ"
+        # mask=None and the fused residual
+        got_n = hip(xd, None)
+        want_n = torch.stack([ref(x[b:b + 1].float(), None)[0] for b in range(batch)])
+        assert_close(got_n, want_n, "mask=None", auto_scale=True)
+        xin = xd.clone()
+        ops.triattn_forward(xin, md, hip._hip_attention_cache, h, starting, residual=xin, out=xin)
+        assert_close(xin, x.float() + want, "residual in place", rel_fro=5e-3, auto_scale=True)
