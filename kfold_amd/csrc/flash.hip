@@ -443,20 +443,24 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
 // ------------------------------------------------------------------------------------------
 // staged kernel (any sequence length, head dim 32 or 64)
 // ------------------------------------------------------------------------------------------
-template <int R, int DKS, int DV>
-__global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(FlashArgs p) {
+// PERROW: every row has its own bias batch (pair-bias attention with a bias per sample, local
+// attention windows); otherwise all rows share bias batch 0.  Queries come in p.nbq blocks of 32
+// per row, keys in p.nb blocks (equal for self attention).
+template <int R, int DKS, int DV, bool PERROW>
+__global__ __launch_bounds__(512, (DKS == 2 ? (PERROW ? 3 : 4) : 2)) void flash_staged_kernel(FlashArgs p) {
     static_assert(DKS == 2 * DV, "head dim = 16*DKS = 32*DV");
     constexpr int A = 2 * R;                       // rows per workgroup
     constexpr int KV_UNITS = DKS * 64;             // 16-byte units of one row's K (or V) block
     constexpr int BIAS_OFF = 2 * A * KV_UNITS;     // unit offset of the bias tiles in a stage
-    constexpr int STAGE_UNITS = BIAS_OFF + 4 * 128;
+    constexpr int BIAS_SETS = PERROW ? A : 1;      // bias tiles of the 4 query blocks, per row or shared
+    constexpr int STAGE_UNITS = BIAS_OFF + BIAS_SETS * 4 * 128;
     constexpr int NLOAD = (STAGE_UNITS + 511) / 512;
     __shared__ __attribute__((aligned(16))) u32x4 stage[2][STAGE_UNITS];
     __shared__ uint8_t cls_s[A][256];              // class of each key block per row
     __shared__ int uniform_s[A];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
-    const int nb = p.nb, H = p.H;
+    const int nb = p.nb, nbq = p.nbq, H = p.H;
     const u32x4* __restrict__ qf = static_cast<const u32x4*>(p.qf);
     const u32x4* __restrict__ kf = static_cast<const u32x4*>(p.kf);
     const u32x4* __restrict__ vf = static_cast<const u32x4*>(p.vf);
@@ -473,13 +477,16 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
     const int h = chunk / rowsets, a0 = (chunk % rowsets) * A;
     const int qbl = wave & 3, rg = wave >> 2;      // this wavefront: query block, row group
     const int qb = qb0 + qbl;
-    const bool wave_active = qb < nb;
-    const int qbc = min(qb, nb - 1);
+    const bool wave_active = qb < nbq;
+    const int qbc = min(qb, nbq - 1);
     const int nr = max(0, min(R, p.nrows - (a0 + rg * R)));   // rows of this wavefront that exist
 
     auto rowc = [&](int ra) { return min(a0 + ra, p.nrows - 1); };                  // clamped row
-    auto blk_units = [&](int a, int blk) -> size_t {
+    auto blk_units = [&](int a, int blk) -> size_t {          // key-side fragments (K, V)
         return (((size_t)a * H + h) * nb + blk) * KV_UNITS;
+    };
+    auto qblk_units = [&](int a, int blk) -> size_t {         // query-side fragments (Q, gate, output)
+        return (((size_t)a * H + h) * nbq + blk) * KV_UNITS;
     };
 
     if (wave < A) {
@@ -499,8 +506,9 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
                 const u32x4* src = region < A ? kf : vf;
                 pre[i] = src[blk_units(rowc(region % A), kb) + off];
             } else if (u < STAGE_UNITS) {
-                const int t = u - BIAS_OFF, q = t >> 7, off = t & 127;
-                pre[i] = bt[(((size_t)h * nb + min(qb0 + q, nb - 1)) * nb + kb) * 128 + off];
+                const int t = u - BIAS_OFF, set = t >> 9, q = (t >> 7) & 3, off = t & 127;
+                const size_t batch = PERROW ? (size_t)rowc(set) : 0;
+                pre[i] = bt[(((batch * H + h) * nbq + min(qb0 + q, nbq - 1)) * nb + kb) * 128 + off];
             }
         }
     };
@@ -522,7 +530,7 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
     for (int r = 0; r < R; ++r) {
         const int a = rowc(rg * R + r);
 #pragma unroll
-        for (int ks = 0; ks < DKS; ++ks) q[r][ks] = as_frag(qf[blk_units(a, qbc) + ks * 64 + lane]);
+        for (int ks = 0; ks < DKS; ++ks) q[r][ks] = as_frag(qf[qblk_units(a, qbc) + ks * 64 + lane]);
         qx[r] = slot0_frag(0.f, half);
 #pragma unroll
         for (int d = 0; d < DV; ++d) o[r][d] = zero;
@@ -542,12 +550,13 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
         if (kb + 1 < nb) prefetch(kb + 1);
         const u32x4* st = stage[kb & 1];
         if (wave_active) {
-            const u32x4 b0 = st[BIAS_OFF + qbl * 128 + lane];
-            const u32x4 b1 = st[BIAS_OFF + qbl * 128 + 64 + lane];
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 if (r >= nr) continue;
                 const int ra = rg * R + r;
+                const int bset = PERROW ? ra : 0;
+                const u32x4 b0 = st[BIAS_OFF + (bset * 4 + qbl) * 128 + lane];
+                const u32x4 b1 = st[BIAS_OFF + (bset * 4 + qbl) * 128 + 64 + lane];
                 int cls = __builtin_amdgcn_readfirstlane((int)cls_s[ra][kb]);
                 const bool uni = uniform_row[r];
                 if (cls & 0x80) {                    // no valid key in this block
@@ -599,7 +608,7 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
         const float inv = fast_rcp(xhalf_sum(l[r]));
 #pragma unroll
         for (int d = 0; d < DV; ++d) {
-            const size_t u0 = blk_units(a, qb) + (2 * d) * 64 + lane;
+            const size_t u0 = qblk_units(a, qb) + (2 * d) * 64 + lane;
             const u32x4 g0 = gf[u0], g1 = gf[u0 + 64];
             f32x16 og;
 #pragma unroll
@@ -619,15 +628,19 @@ __global__ __launch_bounds__(512, (DKS == 2 ? 4 : 2)) void flash_staged_kernel(F
 
 static int launch_staged(FlashArgs p, int head_dim_pad, hipStream_t stream) {
     constexpr int R = 1, A = 2 * R;
-    p.qgroups = (p.nb + 3) / 4;
+    p.qgroups = (p.nbq + 3) / 4;
     p.nchunks = p.H * ((p.nrows + A - 1) / A);
     const int nslots = ((p.nchunks + 7) / 8) * p.qgroups;
-    if (head_dim_pad == 32)
-        hipLaunchKernelGGL((flash_staged_kernel<R, 2, 1>), dim3(nslots * 8), dim3(512), 0, stream, p);
-    else if (head_dim_pad == 64)
-        hipLaunchKernelGGL((flash_staged_kernel<R, 4, 2>), dim3(nslots * 8), dim3(512), 0, stream, p);
-    else
+    const dim3 grid(nslots * 8), block(512);
+    if (head_dim_pad == 32) {
+        if (p.bias_per_row) hipLaunchKernelGGL((flash_staged_kernel<R, 2, 1, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((flash_staged_kernel<R, 2, 1, false>), grid, block, 0, stream, p);
+    } else if (head_dim_pad == 64) {
+        if (p.bias_per_row) hipLaunchKernelGGL((flash_staged_kernel<R, 4, 2, true>), grid, block, 0, stream, p);
+        else hipLaunchKernelGGL((flash_staged_kernel<R, 4, 2, false>), grid, block, 0, stream, p);
+    } else {
         return -1;
+    }
     return 0;
 }
 
@@ -668,28 +681,12 @@ static int launch_strip(FlashArgs p, hipStream_t stream) {
     return 0;
 }
 
-int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream) {
-    if (args.nb > 256) return -1;
-    if (args.bias_per_row) {
-        // a workgroup stages one bias batch: run the rows one at a time
-        for (int a = 0; a < args.nrows; ++a) {
-            FlashArgs one = args;
-            const size_t frag_row = (size_t)args.H * args.nb * (head_dim_pad / 16) * 1024;
-            one.qf = static_cast<const char*>(args.qf) + a * frag_row;
-            one.kf = static_cast<const char*>(args.kf) + a * frag_row;
-            one.vf = static_cast<const char*>(args.vf) + a * frag_row;
-            one.gf = static_cast<const char*>(args.gf) + a * frag_row;
-            one.of = static_cast<char*>(args.of) + a * frag_row;
-            one.biast = static_cast<const char*>(args.biast) + (size_t)a * args.H * args.nb * args.nb * 2048;
-            one.codes = args.codes + (size_t)a * args.nb * 32;
-            one.nrows = 1;
-            one.bias_per_row = 0;
-            const int rc = launch_staged(one, head_dim_pad, stream);
-            if (rc) return rc;
-        }
-        return 0;
-    }
-    if (head_dim_pad == 32 && args.nb <= kStripMaxBlocks && args.nrows >= 4 * kStripWaves)
+int launch_flash(const FlashArgs& args_in, int head_dim_pad, hipStream_t stream) {
+    FlashArgs args = args_in;
+    if (args.nbq <= 0) args.nbq = args.nb;            // self attention
+    if (args.nb > 256 || args.nbq > 256) return -1;
+    if (!args.bias_per_row && args.nbq == args.nb && head_dim_pad == 32 && args.nb <= kStripMaxBlocks &&
+        args.nrows >= 4 * kStripWaves)
         return launch_strip(args, stream);
     return launch_staged(args, head_dim_pad, stream);
 }

@@ -71,9 +71,10 @@ struct TriattnWorkspace {
 struct FlashArgs {
     const void *qf, *kf, *vf, *gf;   // fragment-order operands
     void* of;                         // gated output fragments
-    const void* biast;                // bf16 bias tiles (bias_tile_elem layout)
+    const void* biast;                // bf16 bias tiles [batch][h][query block][key block] (bias_tile_elem layout)
     const uint8_t* codes;             // [nrows][nb*32] key codes
-    int nrows, nb, H;
+    int nrows, nb, H;                 // nb: key blocks of 32 per row
+    int nbq;                          // query blocks per row (0: same as nb, self attention)
     int bias_per_row;                 // 0: one bias for all rows, 1: bias batch index = row
     int qgroups, nchunks;             // filled in by launch_flash
     int rowranges, rows_per_range;    // strip kernel: rows are split into ranges per workgroup
