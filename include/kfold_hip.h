@@ -217,6 +217,39 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
                     int io_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------
+ * Cross attention with pair bias over local windows: the whole
+ * `CrossAttentionPairBias.forward` (model/layers/folding/attention_pair_bias.py:161-260; math of
+ * model/primitives/attention.py:75-94, :239-271) of the atom transformer: W windows, each with
+ * Lq queries (32) attending to Lk keys (128) under its own bias [H, Lq, Lk] and key mask [Lk].
+ * C = channel_a (a multiple of 32), H heads of C/H <= 64 channels, Cs = conditioning channels
+ * (0 = none, else a multiple of 16).  Arithmetic is bf16 MFMA / fp32 accumulation like every
+ * other entry point; the fp32 ("ieee") arithmetic the reference selects for its diffusion
+ * stack (model/model.py:419) is not built.
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_cross_apb_packed_bytes(int C, int H, int Cs);
+
+/* unconditioned: lnq_*, lnk_* [C] (`layernorm_a_q`, `layernorm_a_k`); conditioned: adaq_* / adak_*
+ * are `adaln_a_q` / `adaln_a_k` (`layernorm_s.weight` [Cs], `linear_g` [C, Cs] + bias [C],
+ * `linear_bias` [C, Cs]) and ada_out_* is `linear_ada_out`.  q_w .. o_w [C, C], q_b [C] or NULL. */
+int kfh_cross_apb_pack(const void* lnq_w, const void* lnq_b, const void* lnk_w, const void* lnk_b,
+                       const void* q_w, const void* q_b, const void* k_w, const void* v_w, const void* g_w,
+                       const void* o_w, const void* adaq_s_w, const void* adaq_g_w, const void* adaq_g_b,
+                       const void* adaq_bias_w, const void* adak_s_w, const void* adak_g_w,
+                       const void* adak_g_b, const void* adak_bias_w, const void* ada_out_w,
+                       const void* ada_out_b, int w_dtype, int C, int H, int Cs, void* blob, void* stream);
+
+size_t kfh_cross_apb_workspace_bytes(int W, int Lq, int Lk, int C, int H, int Cs);
+
+/* a_q, out, residual: [W, Lq, C]; a_k: [W, Lk, C]; s_q: [W, Lq, Cs], s_k: [W, Lk, Cs] (Cs > 0);
+ * pair_bias: dense [W, H, Lq, Lk] of bias_dtype; mask: [W, Lk] bytes.
+ * out = (residual or 0) + result; `residual` may alias `out`.  A window whose keys are all
+ * masked attends uniformly over its Lk keys (finite -1e9). */
+int kfh_cross_apb_forward(const void* a_q, const void* a_k, const void* s_q, const void* s_k,
+                          const void* pair_bias, int bias_dtype, const uint8_t* mask, const void* blob,
+                          const void* residual, void* out, void* workspace, size_t workspace_bytes, int W,
+                          int Lq, int Lk, int C, int H, int Cs, float eps, int io_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------
  * Parcae recurrence step of the trunk: replaces the torch line
  *   z = a * z + F.linear(self.layernorm_z(u_t), b)             (model/model.py:528)
  * with a, b from `_parcae_discretized_dynamics` (model/model.py:272-277):

@@ -52,6 +52,11 @@ SIGNATURES: dict[str, tuple] = {
     "kfh_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "kfh_apb_forward": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                 c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+    "kfh_cross_apb_packed_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "kfh_cross_apb_pack": (c_int, [_P] * 20 + [c_int, c_int, c_int, c_int, _P, _P]),
+    "kfh_cross_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "kfh_cross_apb_forward": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_size_t, c_int, c_int,
+                                      c_int, c_int, c_int, c_int, c_float, c_int, _P]),
     "kfh_parcae_packed_bytes": (c_size_t, [c_int]),
     "kfh_parcae_pack": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, _P, _P]),
     "kfh_parcae_step": (c_int, [_P, _P, _P, _P, c_longlong, c_int, c_float, c_int, _P]),

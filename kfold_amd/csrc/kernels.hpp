@@ -128,9 +128,10 @@ int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const floa
 // mask element of (row a, key k) is mask[a * mask_stride + k * key_stride]
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
                       long long mask_stride, hipStream_t stream, long long key_stride = 1);
-// source element (t = batch*H + head, q, k) at t*st + q*sq + k*sk; all zero = dense [.., H, L, L]
+// source element (t = batch*H + head, q, k) at t*st + q*sq + k*sk; all zero = dense [.., H, L, Lk];
+// L queries in nb blocks, Lk keys (0: = L)
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
-                       hipStream_t stream, long long st = 0, long long sq = 0, long long sk = 0);
+                       hipStream_t stream, long long st = 0, long long sq = 0, long long sk = 0, int Lk = 0);
 
 enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS };
 

@@ -102,17 +102,18 @@ void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int 
 
 // Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled bf16 tiles (bias_tile_elem layout);
 // one thread writes the 8 keys of one (tile, chunk, lane) slot.
-// element (t, q, k) of the source is at t * st + q * sq + k * sk (t = batch * H + head)
+// element (t, q, k) of the source is at t * st + q * sq + k * sk (t = batch * H + head); Lq x Lk
+// logits in nbq x nbk tiles
 template <int IO>
 __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __restrict__ tiles,
-                                  long long total, int H, int L, int nb, long long st, long long sq,
-                                  long long sk) {
+                                  long long total, int Lq, int Lk, int nbq, int nbk, long long st,
+                                  long long sq, long long sk) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;      // 16-byte slot
     if (i >= total) return;
     const int lane = (int)(i & 63), c = (int)((i >> 6) & 1);
     long long t = i >> 7;
-    const int kb = (int)(t % nb); t /= nb;
-    const int qb = (int)(t % nb); t /= nb;          // t = batch * H + h
+    const int kb = (int)(t % nbk); t /= nbk;
+    const int qb = (int)(t % nbq); t /= nbq;        // t = batch * H + h
     const int q = qb * 32 + (lane & 31);
     uint32_t w[4];
 #pragma unroll
@@ -122,7 +123,7 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
         for (int u = 0; u < 2; ++u) {
             const int k = kb * 32 + acc_row(8 * c + e + u, lane >> 5);
             float x = 0.f;
-            if (q < L && k < L) {
+            if (q < Lq && k < Lk) {
                 const size_t off = (size_t)(t * st + q * sq + k * sk);
                 if constexpr (IO == KFH_F32) x = static_cast<const float*>(dense)[off];
                 else x = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
@@ -135,16 +136,19 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
 }
 
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
-                       hipStream_t stream, long long st, long long sq, long long sk) {
-    if (st == 0 && sq == 0 && sk == 0) { st = (long long)L * L; sq = L; sk = 1; }    // dense [.., H, L, L]
-    const long long total = (long long)nbatch * H * nb * nb * 128;
+                       hipStream_t stream, long long st, long long sq, long long sk, int Lk) {
+    const int Lq = L, nbq = nb;
+    if (Lk <= 0) Lk = L;
+    const int nbk = (Lk + 31) / 32;
+    if (st == 0 && sq == 0 && sk == 0) { st = (long long)Lq * Lk; sq = Lk; sk = 1; }    // dense [.., H, Lq, Lk]
+    const long long total = (long long)nbatch * H * nbq * nbk * 128;
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, H, L, nb,
-                           st, sq, sk);
+        hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, Lq, Lk, nbq,
+                           nbk, st, sq, sk);
     else
-        hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, H, L, nb,
-                           st, sq, sk);
+        hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, Lq, Lk, nbq,
+                           nbk, st, sq, sk);
 }
 
 }  // namespace kfh

@@ -2,6 +2,7 @@
 
 from .attention_pair_bias import (  # noqa: F401
     AdaLN,
+    CrossAttentionPairBias,
     SelfAttentionPairBias,
     hip_attention_pair_bias,
 )

@@ -7,8 +7,8 @@
 ``attention_pair_bias`` (model/primitives/attention.py:62-66) would call, next to
 ``triton_attention_pair_bias``: it receives already normalised ``x_q``/``x_k``.
 
-Only self attention (``x_q is x_k``, Lq == Lk) is built; the local-window
-``CrossAttentionPairBias`` of the diffusion atom transformer is out of scope.
+``CrossAttentionPairBias`` mirrors the local-window attention of the atom transformer
+(:161-260): Lq queries against Lk keys per window, one bias and key mask per window.
 """
 
 from __future__ import annotations
@@ -146,3 +146,83 @@ class SelfAttentionPairBias(nn.Module):
         else:
             assert s is None
         return _run(self, a, s, pair_bias, mask, apply_norm=True)
+
+
+class CrossAttentionPairBias(nn.Module):
+    """Mirror of the reference's ``CrossAttentionPairBias`` (attention_pair_bias.py:161-260): same
+    constructor, parameter names (``layernorm_a_q`` / ``layernorm_a_k`` or ``adaln_a_q`` /
+    ``adaln_a_k`` + ``linear_ada_out``) and ``forward(a_q, a_k, s_q, s_k, pair_bias, mask)``."""
+
+    def __init__(self, channel_a: int, num_heads: int, channel_s: int | None, inf: float = 1e9,
+                 kernel_backend: str = "hip") -> None:
+        super().__init__()
+        if kernel_backend != "hip":
+            raise ValueError(f"kfold_amd implements kernel_backend='hip' only, got {kernel_backend!r}")
+        assert channel_a % num_heads == 0
+        self.use_single_conditioning = channel_s is not None
+        self.channel_a = channel_a
+        self.channel_s = channel_s
+        self.num_heads = num_heads
+        self.head_dim = channel_a // num_heads
+        self.inf = inf
+        self.kernel_backend = kernel_backend
+        self.linear_q = Linear(channel_a, channel_a, init="default")
+        self.linear_k = LinearNoBias(channel_a, channel_a, init="default")
+        self.linear_v = LinearNoBias(channel_a, channel_a, init="default")
+        self.linear_g = LinearNoBias(channel_a, channel_a, init="gating")
+        self.linear_out = LinearNoBias(channel_a, channel_a,
+                                       init="default" if self.use_single_conditioning else "final")
+        if self.use_single_conditioning:
+            self.adaln_a_q = AdaLN(channel_a, channel_s)
+            self.adaln_a_k = AdaLN(channel_a, channel_s)
+            self.linear_ada_out = Linear(channel_s, channel_a, init="gating")
+            with torch.no_grad():
+                self.linear_ada_out.bias.fill_(-2.0)      # the reference's "gating_closed"
+        else:
+            self.layernorm_a_q = LayerNorm(channel_a, create_offset=True)
+            self.layernorm_a_k = LayerNorm(channel_a, create_offset=True)
+
+    def _weights(self) -> dict:
+        p = dict(q_w=self.linear_q.weight, q_b=self.linear_q.bias, k_w=self.linear_k.weight,
+                 v_w=self.linear_v.weight, g_w=self.linear_g.weight, o_w=self.linear_out.weight)
+        if self.use_single_conditioning:
+            q, k = self.adaln_a_q, self.adaln_a_k
+            p.update(adaq_s_w=q.layernorm_s.weight, adaq_g_w=q.linear_g.weight, adaq_g_b=q.linear_g.bias,
+                     adaq_bias_w=q.linear_bias.weight, adak_s_w=k.layernorm_s.weight,
+                     adak_g_w=k.linear_g.weight, adak_g_b=k.linear_g.bias, adak_bias_w=k.linear_bias.weight,
+                     ada_out_w=self.linear_ada_out.weight, ada_out_b=self.linear_ada_out.bias)
+        else:
+            p.update(lnq_w=self.layernorm_a_q.weight, lnq_b=self.layernorm_a_q.bias,
+                     lnk_w=self.layernorm_a_k.weight, lnk_b=self.layernorm_a_k.bias)
+        return p
+
+    @torch.compiler.disable
+    def forward(self, a_q: torch.Tensor, a_k: torch.Tensor, s_q: torch.Tensor | None,
+                s_k: torch.Tensor | None, pair_bias: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
+        """a_q [..., W, Lq, c_a], a_k [..., W, Lk, c_a], s_q / s_k [..., W, L., c_s] or None,
+        pair_bias [..., W, H, Lq, Lk], mask [..., W, Lk] -> [..., W, Lq, c_a]."""
+        check_inference(a_q, "cross attention with pair bias")
+        check_inf(self)
+        if self.use_single_conditioning:
+            assert s_q is not None and s_k is not None
+        else:
+            assert s_q is None and s_k is None
+        if self.linear_g.bias is not None or self.linear_out.bias is not None:
+            raise NotImplementedError("hip cross attention: gate / output projection biases")
+        w = self._weights()
+        cs = self.channel_s or 0
+        blob = cached_blob(self, "_hip_cross_cache", cache_key(tuple(w.values()), a_q, torch.bfloat16),
+                           lambda: ops.cross_apb_pack(self.channel_a, self.num_heads, cs, a_q.device, **w))
+        lead = a_q.shape[:-2]
+        Lq, Lk = a_q.shape[-2], a_k.shape[-2]
+        io = a_q if a_q.dtype in (torch.bfloat16, torch.float32) else a_q.float()
+
+        def flat(t, keep):
+            full = torch.broadcast_to(t, tuple(lead) + t.shape[t.dim() - keep:])
+            return full.reshape((-1,) + t.shape[t.dim() - keep:])
+
+        eps = (self.adaln_a_q.layernorm_a.eps if self.use_single_conditioning else self.layernorm_a_q.eps)
+        out = ops.cross_apb_forward(io.reshape(-1, Lq, self.channel_a), flat(a_k, 2),
+                                    None if s_q is None else flat(s_q, 2), None if s_k is None else flat(s_k, 2),
+                                    flat(pair_bias, 3), flat(mask, 1), blob, self.num_heads, cs, eps=eps)
+        return out.reshape(a_q.shape).to(a_q.dtype)

@@ -351,3 +351,62 @@ def parcae_step(z: torch.Tensor, u: torch.Tensor, blob: torch.Tensor, eps: float
         check(L.kfh_parcae_step(z.data_ptr(), u.data_ptr(), blob.data_ptr(), out.data_ptr(), rows, C,
                                 float(eps), _io_dtype(z), _stream(dev)))
     return out
+
+
+# ---------------------------------------------------------------------------------------
+# cross attention with pair bias over local windows
+# ---------------------------------------------------------------------------------------
+_CROSS_ORDER = ("lnq_w", "lnq_b", "lnk_w", "lnk_b", "q_w", "q_b", "k_w", "v_w", "g_w", "o_w", "adaq_s_w",
+                "adaq_g_w", "adaq_g_b", "adaq_bias_w", "adak_s_w", "adak_g_w", "adak_g_b", "adak_bias_w",
+                "ada_out_w", "ada_out_b")
+
+
+def cross_apb_pack(C: int, H: int, Cs: int, device: torch.device, **weights) -> torch.Tensor:
+    L = _lib.lib()
+    nbytes = L.kfh_cross_apb_packed_bytes(C, H, Cs)
+    if nbytes == 0:
+        raise NotImplementedError(f"hip cross attention: C={C}, H={H}, Cs={Cs} unsupported")
+    ws = _weights_f32(device, *[weights.get(k) for k in _CROSS_ORDER])
+    blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        check(L.kfh_cross_apb_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, Cs, blob.data_ptr(), _stream(device)))
+    return blob
+
+
+def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias: torch.Tensor, mask: torch.Tensor,
+                      blob: torch.Tensor, heads: int, cond_channels: int, eps: float = 1e-5,
+                      residual: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
+    """a_q [W, Lq, C], a_k [W, Lk, C], s_q / s_k [W, L., Cs] or None, pair_bias [W, H, Lq, Lk], mask [W, Lk]."""
+    dev = _require_cuda(a_q, a_k, s_q, s_k, pair_bias, mask, blob, residual, out)
+    W, Lq, C = a_q.shape
+    Lk = a_k.shape[1]
+    if a_k.shape != (W, Lk, C) or pair_bias.shape != (W, heads, Lq, Lk) or mask.shape != (W, Lk):
+        raise ValueError("cross attention: inconsistent window shapes")
+    aq, ak = a_q.contiguous(), a_k.contiguous().to(a_q.dtype)
+    pb = pair_bias.contiguous()
+    if pb.dtype not in _IO_DTYPES:
+        pb = pb.float()
+    m8 = _mask_bytes(mask, mask.shape)
+    sq = sk = None
+    if cond_channels:
+        sq, sk = s_q.contiguous().to(aq.dtype), s_k.contiguous().to(aq.dtype)
+        if sq.shape != (W, Lq, cond_channels) or sk.shape != (W, Lk, cond_channels):
+            raise ValueError("cross attention: conditioning shapes do not match")
+    if out is None:
+        out = torch.empty_like(aq)
+    elif out.shape != a_q.shape or out.dtype != a_q.dtype or not out.is_contiguous():
+        raise ValueError("out must be contiguous with the shape and dtype of a_q")
+    if residual is not None and (residual.shape != a_q.shape or residual.dtype != a_q.dtype
+                                 or not residual.is_contiguous()):
+        raise ValueError("residual must be contiguous with the shape and dtype of a_q")
+    L = _lib.lib()
+    ws_bytes = L.kfh_cross_apb_workspace_bytes(W, Lq, Lk, C, heads, cond_channels)
+    if ws_bytes == 0:
+        raise NotImplementedError(f"hip cross attention: unsupported shape W={W} Lq={Lq} Lk={Lk} C={C} H={heads}")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    with torch.cuda.device(dev):
+        check(L.kfh_cross_apb_forward(aq.data_ptr(), ak.data_ptr(), _ptr(sq), _ptr(sk), pb.data_ptr(),
+                                      _io_dtype(pb), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
+                                      out.data_ptr(), ws.data_ptr(), ws_bytes, W, Lq, Lk, C, heads,
+                                      cond_channels, float(eps), _io_dtype(aq), _stream(dev)))
+    return out

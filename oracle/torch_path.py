@@ -318,6 +318,47 @@ class SelfAttentionPairBias(nn.Module):
         return a
 
 
+class CrossAttentionPairBias(nn.Module):
+    """model/layers/folding/attention_pair_bias.py:161-260 — attention of Lq queries over Lk
+    keys inside local windows (leading dims ..., W), each side with its own LayerNorm / AdaLN."""
+
+    def __init__(self, channel_a: int, num_heads: int, channel_s: int | None, inf: float = 1e9,
+                 kernel_backend: str = "torch"):
+        super().__init__()
+        assert channel_a % num_heads == 0
+        self.channel_a = channel_a
+        self.num_heads = num_heads
+        self.head_dim = channel_a // num_heads
+        self.inf = inf
+        self.kernel_backend = kernel_backend
+        self.use_single_conditioning = channel_s is not None
+        self.linear_q = Linear(channel_a, channel_a)
+        self.linear_k = LinearNoBias(channel_a, channel_a)
+        self.linear_v = LinearNoBias(channel_a, channel_a)
+        self.linear_g = LinearNoBias(channel_a, channel_a)
+        self.linear_out = LinearNoBias(channel_a, channel_a)
+        if self.use_single_conditioning:
+            self.adaln_a_q = AdaLN(channel_a, channel_s)
+            self.adaln_a_k = AdaLN(channel_a, channel_s)
+            self.linear_ada_out = Linear(channel_s, channel_a)
+        else:
+            self.layernorm_a_q = LayerNorm(channel_a)
+            self.layernorm_a_k = LayerNorm(channel_a)
+
+    def forward(self, a_q, a_k, s_q, s_k, pair_bias, mask):
+        if self.use_single_conditioning:                                          # :241-244
+            a_q = self.adaln_a_q(a_q, s_q)
+            a_k = self.adaln_a_k(a_k, s_k)
+        else:                                                                     # :245-248
+            assert s_q is None and s_k is None
+            a_q = self.layernorm_a_q(a_q)
+            a_k = self.layernorm_a_k(a_k)
+        a_q = torch_attention_pair_bias(self, a_q, a_k, pair_bias, mask)          # :250-258
+        if self.use_single_conditioning:                                          # :260-262
+            a_q = torch.sigmoid(self.linear_ada_out(s_q)) * a_q
+        return a_q
+
+
 # ---------------------------------------------------------------------------
 # blocks
 # ---------------------------------------------------------------------------

@@ -265,3 +265,31 @@ def test_parcae_step_vs_brute_and_closed_forms():
     with torch.no_grad():
         f.parcae_log_delta.fill_(-40.0)
     assert torch.allclose(f(zz, uu), zz, atol=1e-12)
+
+
+def test_cross_apb_windows_vs_brute():
+    """Lq != Lk, one bias and one key mask per window, each side with its own norm."""
+    m = _rand_init(O.CrossAttentionPairBias(6, 2, None), 41)
+    W, Lq, Lk = 3, 2, 5
+    aq, ak = _rand((W, Lq, 6), 42), _rand((W, Lk, 6), 43)
+    bias = _rand((W, 2, Lq, Lk), 44)
+    mask = torch.rand(W, Lk, generator=torch.Generator().manual_seed(45)) > 0.3
+    mask[:, 0] = True
+    got = m(aq, ak, None, None, bias, mask).detach().numpy()
+    p = _np_params(m)
+    for w in range(W):
+        qn = np.array([brute._ln(r, p["layernorm_a_q.weight"], p["layernorm_a_q.bias"]) for r in aq[w].numpy()])
+        kn = np.array([brute._ln(r, p["layernorm_a_k.weight"], p["layernorm_a_k.bias"]) for r in ak[w].numpy()])
+        want = brute.attention_pair_bias(qn, kn, bias[w].numpy(), mask[w].numpy(), p, heads=2)
+        assert np.allclose(got[w], want, atol=1e-9)
+    # conditioned wiring: AdaLN per side, sigmoid(linear_ada_out(s_q)) gate on the result
+    c = _rand_init(O.CrossAttentionPairBias(6, 2, 4), 46)
+    sq, sk = _rand((W, Lq, 4), 47), _rand((W, Lk, 4), 48)
+    got = c(aq, ak, sq, sk, bias, mask)
+    qn, kn = c.adaln_a_q(aq, sq), c.adaln_a_k(ak, sk)
+    core = O.torch_attention_pair_bias(c, qn, kn, bias, mask)
+    assert torch.allclose(got, torch.sigmoid(c.linear_ada_out(sq)) * core, atol=1e-12)
+    pc = _np_params(c)
+    want0 = brute.attention_pair_bias(qn[0].detach().numpy(), kn[0].detach().numpy(), bias[0].numpy(),
+                                      mask[0].numpy(), pc, heads=2)
+    assert np.allclose(core[0].detach().numpy(), want0, atol=1e-9)

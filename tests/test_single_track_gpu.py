@@ -149,3 +149,43 @@ def test_apb_diffusion_variant(s_shared):
         got = hip(a.to(DEV), s.to(DEV), bias.to(DEV), mask.to(DEV))
     assert got.shape == a.shape and got.dtype == a.dtype
     assert_close(got, want, "apb diffusion variant", auto_scale=True)
+
+
+@pytest.mark.parametrize("cond", [False, True])
+def test_cross_attention_local_windows(cond):
+    """The atom transformer's attention: windows of 32 queries x 128 keys, c_atom 128, 4 heads x 32,
+    one bias and key mask per window, 5 samples; with and without single conditioning."""
+    from kfold_amd.layers import CrossAttentionPairBias
+    from oracle import torch_path as O
+
+    print(f"case cross attention windows cond={cond}", flush=True)
+    cs = 128 if cond else None
+    ref, hip = _pair(O.CrossAttentionPairBias, CrossAttentionPairBias, (128, 4, cs), seed=12, std=0.05,
+                     tweak=_affine)
+    S, W, Lq, Lk = 5, 23, 32, 128
+    g = torch.Generator().manual_seed(14)
+    aq = torch.randn(S, W, Lq, 128, generator=g).bfloat16()
+    ak = torch.randn(S, W, Lk, 128, generator=g).bfloat16()
+    sq = torch.randn(S, W, Lq, 128, generator=g).bfloat16() if cond else None
+    sk = torch.randn(S, W, Lk, 128, generator=g).bfloat16() if cond else None
+    bias = torch.randn(1, W, 4, Lq, Lk, generator=g)              # shared by the samples
+    mask = torch.rand(1, W, Lk, generator=g) > 0.2
+    mask[0, 3] = False                                            # a window with every key masked
+    mask[0, 7, 40:] = False
+    f = lambda t: None if t is None else t.float()
+    with torch.no_grad():
+        want = ref(aq.float(), ak.float(), f(sq), f(sk), bias, mask)
+        d = lambda t: None if t is None else t.to(DEV)
+        got = hip(aq.to(DEV), ak.to(DEV), d(sq), d(sk), bias.to(DEV), mask.to(DEV))
+    assert got.shape == aq.shape and got.dtype == aq.dtype
+    print(assert_close(got, want, "cross attention windows", auto_scale=True), flush=True)
+    # odd window shape: 20 queries, 70 keys
+    Lq2, Lk2 = 20, 70
+    aq2, ak2 = aq[:1, :, :Lq2].contiguous(), ak[:1, :, :Lk2].contiguous()
+    sq2 = None if sq is None else sq[:1, :, :Lq2].contiguous()
+    sk2 = None if sk is None else sk[:1, :, :Lk2].contiguous()
+    b2, m2 = bias[:, :, :, :Lq2, :Lk2].contiguous(), mask[:, :, :Lk2].contiguous()
+    with torch.no_grad():
+        want2 = ref(aq2.float(), ak2.float(), f(sq2), f(sk2), b2, m2)
+        got2 = hip(aq2.to(DEV), ak2.to(DEV), d(sq2), d(sk2), b2.to(DEV), m2.to(DEV))
+    assert_close(got2, want2, "cross attention, 20 x 70 windows", auto_scale=True)
