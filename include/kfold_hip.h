@@ -264,10 +264,12 @@ size_t kfh_parcae_packed_bytes(int C);
 int kfh_parcae_pack(const void* ln_w, const void* ln_b, const void* log_a, const void* log_delta,
                     const void* b_cont, int w_dtype, int C, void* blob, void* stream);
 
-/* out[r,:] = a * z[r,:] + b LN(u[r,:]) for r < rows; z, u, out: [rows, C] (io_dtype).
- * `out` may alias `z` (the in-place update of the pair state); it must not alias `u`. */
-int kfh_parcae_step(const void* z, const void* u, const void* blob, void* out, long long rows, int C,
-                    float eps, int io_dtype, void* stream);
+/* out[r,:] = a * z[r,:] + b LN(u[r,:] + u_add[r,:]) for r < rows; z, u, u_add, out: [rows, C]
+ * (io_dtype).  `u_add` may be NULL; with it the sum `u_t = z_inputs + lm_stack(...)` of
+ * model/model.py:526 never goes through memory.  `out` may alias `z` (the in-place update of
+ * the pair state); it must not alias `u` or `u_add`. */
+int kfh_parcae_step(const void* z, const void* u, const void* u_add, const void* blob, void* out,
+                    long long rows, int C, float eps, int io_dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -59,7 +59,7 @@ SIGNATURES: dict[str, tuple] = {
                                       c_int, c_int, c_int, c_int, c_float, c_int, _P]),
     "kfh_parcae_packed_bytes": (c_size_t, [c_int]),
     "kfh_parcae_pack": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, _P, _P]),
-    "kfh_parcae_step": (c_int, [_P, _P, _P, _P, c_longlong, c_int, c_float, c_int, _P]),
+    "kfh_parcae_step": (c_int, [_P, _P, _P, _P, _P, c_longlong, c_int, c_float, c_int, _P]),
 }
 
 _lib = None

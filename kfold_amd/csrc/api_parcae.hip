@@ -28,15 +28,15 @@ int kfh_parcae_pack(const void* ln_w, const void* ln_b, const void* log_a, const
     return check_launch("parcae_pack");
 }
 
-int kfh_parcae_step(const void* z, const void* u, const void* blob, void* out, long long rows, int C,
-                    float eps, int io_dtype, void* stream) {
+int kfh_parcae_step(const void* z, const void* u, const void* u_add, const void* blob, void* out,
+                    long long rows, int C, float eps, int io_dtype, void* stream) {
     if (C != 128 && C != 256) return fail(KFH_EUNSUPPORTED, "parcae_step: C=%d, built for C=128 and C=256", C);
     if (rows < 0) return fail(KFH_EINVAL, "parcae_step: rows=%lld", rows);
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "parcae_step: bad io_dtype %d", io_dtype);
     if (!z || !u || !blob || !out) return fail(KFH_EINVAL, "parcae_step: null pointer argument");
-    if (out == u) return fail(KFH_EINVAL, "parcae_step: out may alias z, not u");
+    if (out == u || (u_add && out == u_add)) return fail(KFH_EINVAL, "parcae_step: out may alias z, not u");
     if (rows == 0) return KFH_OK;
-    if (launch_parcae_step(z, u, io_dtype, static_cast<const char*>(blob), out, rows, C, eps,
+    if (launch_parcae_step(z, u, u_add, io_dtype, static_cast<const char*>(blob), out, rows, C, eps,
                            static_cast<hipStream_t>(stream)) != 0)
         return fail(KFH_EUNSUPPORTED, "parcae_step: shape not built (rows=%lld C=%d)", rows, C);
     return check_launch("parcae_step");

@@ -211,9 +211,11 @@ __device__ __forceinline__ bf16x8 lds_frag_c(const char* tile, int row, int ks, 
     return *reinterpret_cast<const bf16x8*>(tile + row * xs_bytes<C>() + ks * 32 + half * 16);
 }
 
+// `src2` (may be null) is a second tensor of the same layout that is added before normalising.
 template <int IO, int ROWS, int C, class RowOff, int NTHREADS = 256>
 __device__ __forceinline__ void stage_ln_rows_c(char* tile, const void* src, const float* lnp,
-                                                float eps, int tid, RowOff row_off) {
+                                                float eps, int tid, RowOff row_off,
+                                                const void* src2 = nullptr) {
     constexpr int NJ = C / 128;
     constexpr int RG = NTHREADS / 16, NIT = ROWS / RG;
     const int r16 = tid >> 4, ch = tid & 15;
@@ -232,6 +234,15 @@ __device__ __forceinline__ void stage_ln_rows_c(char* tile, const void* src, con
 #pragma unroll
             for (int j = 0; j < NJ; ++j)
                 load8<IO>(src, (size_t)(valid[it] ? off : 0) + 128 * j + ch * 8, x[it][j]);
+            if (src2) {
+#pragma unroll
+                for (int j = 0; j < NJ; ++j) {
+                    float y[8];
+                    load8<IO>(src2, (size_t)(valid[it] ? off : 0) + 128 * j + ch * 8, y);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) x[it][j][i] += y[i];
+                }
+            }
         }
 #pragma unroll
         for (int it = 0; it < GROUP; ++it) {

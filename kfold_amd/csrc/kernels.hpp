@@ -118,8 +118,8 @@ void launch_pair_bias(const void* z, int io_dtype, const char* blob, uint16_t* t
 inline size_t parcae_blob_bytes(int C) { return (size_t)C * C * 2 + 3 * (size_t)C * 4 + (size_t)C * C * 4; }
 void launch_parcae_dynamics(const void* log_a, const void* log_delta, const void* b_cont, int wdtype,
                             float* a_out, float* b_out, int C, hipStream_t stream);
-int launch_parcae_step(const void* z, const void* u, int io_dtype, const char* blob, void* out, long long M,
-                       int C, float eps, hipStream_t stream);
+int launch_parcae_step(const void* z, const void* u, const void* u2, int io_dtype, const char* blob, void* out,
+                       long long M, int C, float eps, hipStream_t stream);
 
 // ---- single-track helpers (rows.hip, linear.hip) -------------------------------------------
 // transpose_n > 0: the M = n*n rows are written transposed as an [n, n] grid of rows

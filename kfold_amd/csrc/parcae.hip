@@ -2,6 +2,7 @@
 // discretised dynamics of :272-277):
 //     delta = softplus(log_delta);  a = exp(-delta * exp(log_a));  B = delta[:, None] * b_cont
 //     z <- a * z + B LN(u)                      (F.linear: B is [out, in]; LN = layernorm_z)
+// with u = u1 + u2 when a second input is given (u_t = z_inputs + lm_stack(...), :526).
 // One pass: u rows are LayerNorm-ed into LDS, multiplied with the packed B on the matrix cores
 // and added to a * z in the store epilogue.  HBM-bound: reads z and u, writes z.
 #include "kernels.hpp"
@@ -30,6 +31,7 @@ __global__ void parcae_dynamics_kernel(const void* __restrict__ log_a, const voi
 // ROW_INTERLEAVE4: block nb, lane col <-> channel 128*g + 4*col + nb).
 template <int IO, int C>
 __global__ __launch_bounds__(256, 3) void parcae_step_kernel(const void* z, const void* __restrict__ u,
+                                                             const void* __restrict__ u2,
                                                              const char* __restrict__ blob, void* out,
                                                              long long M, float eps) {
     constexpr int KS = C / 16;
@@ -44,7 +46,7 @@ __global__ __launch_bounds__(256, 3) void parcae_step_kernel(const void* z, cons
         const long long p = p0 + row;
         return p < M ? p * C : -1;
     };
-    stage_ln_rows_c<IO, 128, C, decltype(row_off), 256>(smem, u, lnp, eps, tid, row_off);
+    stage_ln_rows_c<IO, 128, C, decltype(row_off), 256>(smem, u, lnp, eps, tid, row_off, u2);
     __syncthreads();
     bf16x8 xf[KS];
 #pragma unroll
@@ -109,13 +111,13 @@ void launch_parcae_dynamics(const void* log_a, const void* log_delta, const void
                            log_delta, b_cont, a_out, b_out, C);
 }
 
-int launch_parcae_step(const void* z, const void* u, int io_dtype, const char* blob, void* out, long long M,
-                       int C, float eps, hipStream_t stream) {
+int launch_parcae_step(const void* z, const void* u, const void* u2, int io_dtype, const char* blob, void* out,
+                       long long M, int C, float eps, hipStream_t stream) {
     if (M <= 0) return 0;
     if (M > 0x7fffffffLL * 128) return -1;
     dim3 grid((unsigned)((M + 127) / 128)), block(256);
 #define KFH_PARCAE(IO, CC) \
-    hipLaunchKernelGGL((parcae_step_kernel<IO, CC>), grid, block, 0, stream, z, u, blob, out, M, eps)
+    hipLaunchKernelGGL((parcae_step_kernel<IO, CC>), grid, block, 0, stream, z, u, u2, blob, out, M, eps)
     if (C == 128) {
         if (io_dtype == KFH_F32) KFH_PARCAE(KFH_F32, 128); else KFH_PARCAE(KFH_BF16, 128);
     } else if (C == 256) {

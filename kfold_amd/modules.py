@@ -181,11 +181,63 @@ class ParcaeStep(nn.Module):
         self.parcae_log_delta = nn.Parameter(torch.full((channel_z,), math.log(math.expm1(delta_init))))
         self.parcae_b_cont = nn.Parameter(torch.eye(channel_z))
 
-    def forward(self, z: torch.Tensor, u: torch.Tensor, inplace: bool = True) -> torch.Tensor:
+    def forward(self, z: torch.Tensor, u: torch.Tensor, inplace: bool = True,
+                u_add: torch.Tensor | None = None) -> torch.Tensor:
+        """``a * z + B LN(u [+ u_add])``."""
         check_inference(z, "Parcae step")
         _contiguous_io(z, "z")
         params = (self.layernorm_z.weight, self.layernorm_z.bias, self.parcae_log_a, self.parcae_log_delta,
                   self.parcae_b_cont)
         blob = cached_blob(self, "_hip_parcae_cache", cache_key(params, z, torch.bfloat16),
                            lambda: ops.parcae_pack(*params, device=z.device))
-        return ops.parcae_step(z, u.contiguous(), blob, eps=self.layernorm_z.eps, out=z if inplace else None)
+        return ops.parcae_step(z, u.contiguous(), blob, eps=self.layernorm_z.eps, out=z if inplace else None,
+                               u_add=u_add)
+
+
+class TrianglularStack(nn.Module):
+    """A stack of ``TriangularBlock`` (reference: model/modules/tri_stack.py:31-93, same spelling
+    and the same ``blocks`` list, so its state-dict keys are the reference's)."""
+
+    def __init__(self, channel_z: int = 256, num_blocks: int = 48, dropout: float = 0.25,
+                 blocks_per_ckpt: int | None = None, kernel_backend: str = "hip"):
+        super().__init__()
+        self.kernel_backend = kernel_backend
+        self.channel_z = channel_z
+        self.num_blocks = num_blocks
+        self.blocks = nn.ModuleList(TriangularBlock(channel_z, dropout, kernel_backend=kernel_backend)
+                                    for _ in range(num_blocks))
+
+    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor) -> torch.Tensor:
+        """z is updated in place block after block (the reference's eval-mode adds)."""
+        for blk in self.blocks:
+            z = blk(z, pair_mask)
+        return z
+
+
+class ParcaeTrunk(ParcaeStep):
+    """The pair-state recurrence of ``KFold.run_trunk`` (model/model.py:522-529) on the hip backend:
+
+        for each recycle:  u = z_inputs + lm_stack(z_lm);  z = a * z + B LN(u);  z = main_stack(z)
+
+    Sub-modules and parameters carry the names they have on the reference's ``KFold`` (``lm_stack``,
+    ``main_stack``, ``layernorm_z``, ``parcae_log_a``, ``parcae_log_delta``, ``parcae_b_cont``), so
+    ``load_reference_weights`` fills them from a KFold state dict.  The reference draws a fresh
+    dropout mask on ``z_lm`` every recycle (:525); pass the already dropped-out tensor (or a
+    callable returning it) as ``z_lm``."""
+
+    def __init__(self, channel_z: int = 256, lm_blocks: int = 4, main_blocks: int = 48,
+                 decay_init: float = 0.4472135954999579, kernel_backend: str = "hip"):
+        super().__init__(channel_z, decay_init, kernel_backend)
+        self.lm_stack = TrianglularStack(channel_z, lm_blocks, kernel_backend=kernel_backend)
+        self.main_stack = TrianglularStack(channel_z, main_blocks, kernel_backend=kernel_backend)
+
+    def forward(self, z: torch.Tensor, z_inputs: torch.Tensor, z_lm, pair_mask: torch.Tensor,
+                num_recycles: int = 0) -> torch.Tensor:
+        """z [B, N, N, C] (the pair state, updated in place), z_inputs [B, N, N, C], z_lm a tensor
+        or a callable giving this recycle's (dropped-out) LM pair embedding."""
+        for _ in range(num_recycles + 1):
+            lm_in = z_lm() if callable(z_lm) else z_lm
+            lm = self.lm_stack(lm_in.clone(), pair_mask)          # the stack works in place
+            ParcaeStep.forward(self, z, lm, inplace=True, u_add=z_inputs.contiguous())
+            z = self.main_stack(z, pair_mask)
+        return z

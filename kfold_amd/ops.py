@@ -331,11 +331,13 @@ def parcae_pack(ln_w, ln_b, log_a, log_delta, b_cont, device: torch.device) -> t
 
 
 def parcae_step(z: torch.Tensor, u: torch.Tensor, blob: torch.Tensor, eps: float = 1e-5,
-                out: torch.Tensor | None = None) -> torch.Tensor:
-    """``out = a * z + b LN(u)`` over the last dim; ``out`` may be ``z`` (in place)."""
-    dev = _require_cuda(z, u, blob, out)
+                out: torch.Tensor | None = None, u_add: torch.Tensor | None = None) -> torch.Tensor:
+    """``out = a * z + b LN(u [+ u_add])`` over the last dim; ``out`` may be ``z`` (in place)."""
+    dev = _require_cuda(z, u, blob, out, u_add)
     if u.shape != z.shape or u.dtype != z.dtype:
         raise ValueError("z and u must have the same shape and dtype")
+    if u_add is not None and (u_add.shape != z.shape or u_add.dtype != z.dtype or not u_add.is_contiguous()):
+        raise ValueError("u_add must be contiguous with the shape and dtype of z")
     C = z.shape[-1]
     rows = z.numel() // C if z.numel() else 0
     if not z.is_contiguous() or not u.is_contiguous():
@@ -348,7 +350,7 @@ def parcae_step(z: torch.Tensor, u: torch.Tensor, blob: torch.Tensor, eps: float
         return out
     L = _lib.lib()
     with torch.cuda.device(dev):
-        check(L.kfh_parcae_step(z.data_ptr(), u.data_ptr(), blob.data_ptr(), out.data_ptr(), rows, C,
+        check(L.kfh_parcae_step(z.data_ptr(), u.data_ptr(), _ptr(u_add), blob.data_ptr(), out.data_ptr(), rows, C,
                                 float(eps), _io_dtype(z), _stream(dev)))
     return out
 

@@ -492,3 +492,35 @@ class ParcaeStep(nn.Module):
     def forward(self, z: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
         a, b = self.dynamics()
         return a * z + F.linear(self.layernorm_z(u), b)              # :528
+
+
+class TrianglularStack(nn.Module):
+    """model/modules/tri_stack.py:31-93 (plain loop at inference)."""
+
+    def __init__(self, channel_z: int = 256, num_blocks: int = 48):
+        super().__init__()
+        self.blocks = nn.ModuleList(TriangularBlock(channel_z) for _ in range(num_blocks))
+
+    def forward(self, z, pair_mask):
+        for blk in self.blocks:
+            z = blk(z, pair_mask)
+        return z
+
+
+class ParcaeTrunk(ParcaeStep):
+    """The recurrence of ``KFold.run_trunk`` (model/model.py:522-529) with the dropout on ``z_lm``
+    (:525) left to the caller."""
+
+    def __init__(self, channel_z: int = 256, lm_blocks: int = 4, main_blocks: int = 48,
+                 decay_init: float = 0.4472135954999579):
+        super().__init__(channel_z, decay_init)
+        self.lm_stack = TrianglularStack(channel_z, lm_blocks)
+        self.main_stack = TrianglularStack(channel_z, main_blocks)
+
+    def forward(self, z, z_inputs, z_lm, pair_mask, num_recycles: int = 0):
+        a, b = self.dynamics()
+        for _ in range(num_recycles + 1):
+            u_t = z_inputs + self.lm_stack(z_lm.clone(), pair_mask)              # :526
+            z = a * z + F.linear(self.layernorm_z(u_t), b)                        # :528
+            z = self.main_stack(z, pair_mask)                                     # :529
+        return z

@@ -70,3 +70,44 @@ def test_parcae_module_names_and_errors():
     z = torch.zeros(4, 128, device=DEV)
     with torch.no_grad(), pytest.raises(ValueError):
         hip(z, torch.zeros(4, 64, device=DEV))
+
+
+def test_parcae_trunk_recurrence_and_reference_named_weights():
+    """Two recycles of the trunk recurrence at c_z = 256 (2 + 3 triangular blocks), weights loaded
+    from a state dict that carries the reference model's key names."""
+    from kfold_amd import modules as M
+    from kfold_amd.runtime import load_reference_weights
+    from oracle import torch_path as O
+
+    print("case parcae trunk", flush=True)
+    C, n = 256, 40
+    ref = O.ParcaeTrunk(C, lm_blocks=2, main_blocks=3).eval()
+    synthetic.init_weights_(ref, 21)
+    with torch.no_grad():
+        ref.parcae_b_cont.copy_(torch.eye(C) + 0.05 * torch.randn(C, C, generator=torch.Generator().manual_seed(2)))
+        ref.parcae_log_a.zero_()
+        ref.parcae_log_delta.fill_(0.2)
+    # a checkpoint of the whole model: the trunk's entries sit beside ones with no hip counterpart
+    ckpt = {k: v.clone() for k, v in ref.state_dict().items()}
+    ckpt["input_embedder.linear.weight"] = torch.zeros(3, 3)
+    ckpt["refine_stack.blocks.0.tri_mul_out.linear_p_in.weight"] = torch.zeros(2 * C, C)
+    hip = M.ParcaeTrunk(C, lm_blocks=2, main_blocks=3).eval()
+    used = load_reference_weights(hip, ckpt)
+    assert "main_stack.blocks.2.transition_z.linear_out.weight" in used and len(used) == len(hip.state_dict())
+    with pytest.raises(KeyError):
+        load_reference_weights(M.TrianglularStack(C, 1), ckpt, prefix="no_such_stack.")
+    sub = M.TrianglularStack(C, 3).eval()
+    load_reference_weights(sub, ckpt, prefix="main_stack.")
+    assert torch.equal(sub.blocks[1].tri_mul_in.linear_g_in.weight, ref.main_stack.blocks[1].tri_mul_in.linear_g_in.weight)
+    hip.to(DEV)
+    g = torch.Generator().manual_seed(5)
+    z0 = (0.3 * torch.randn(1, n, n, C, generator=g))
+    zin = torch.randn(1, n, n, C, generator=g)
+    zlm = torch.randn(1, n, n, C, generator=g)
+    pm = synthetic.pair_mask_from_tokens(synthetic.token_mask(n, 5))
+    with torch.no_grad():
+        want = ref(z0.clone(), zin, zlm, pm.float(), num_recycles=1)
+        got = hip(z0.to(DEV), zin.to(DEV), zlm.to(DEV), pm.to(DEV), num_recycles=1)
+    # a wiring test, not a benchmark configuration: 12 chained stages on an O(1) state, so the
+    # absolute limits scale with the state's RMS; the relative gate is the sharp one
+    print(assert_close(got, want, "parcae trunk, fp32 stream, 2 recycles", rel_fro=8e-3, auto_scale=True), flush=True)
