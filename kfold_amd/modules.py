@@ -40,11 +40,12 @@ def _contiguous_io(t: torch.Tensor, name: str) -> None:
         raise TypeError(f"{name}: the hip block runs on bfloat16 or float32 tensors, got {t.dtype}")
 
 
-def _trimul_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None:
+def _trimul_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor, before_write=None) -> None:
     params = _tm_parameters(mod)
     blob = cached_blob(mod, "_hip_multiplication_cache", cache_key(params, z, torch.bfloat16),
                        lambda: ops.trimul_pack(*params, device=z.device))
-    ops.trimul_forward(z, mask, blob, mod.direction, eps=mod.layernorm_in.eps, residual=z, out=z)
+    ops.trimul_forward(z, mask, blob, mod.direction, eps=mod.layernorm_in.eps, residual=z, out=z,
+                       before_write=before_write)
 
 
 def _triattn_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None:
@@ -72,15 +73,17 @@ class PairformerBlock(nn.Module):
                                                        kernel_backend=kernel_backend)
         self.transition_z = Transition(channel_z, expansion_factor=2)
 
-    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor, inplace_output: bool = False) -> torch.Tensor:
+    def forward(self, z: torch.Tensor, pair_mask: torch.Tensor, inplace_output: bool = False,
+                before_first_write=None) -> torch.Tensor:
         """z [B, N, N, C] is updated in place by the four triangle ops (as the reference does in
         eval mode); returns ``(z + transition(z)) * pair_mask`` as a new tensor, or written over
-        ``z`` when ``inplace_output`` is set."""
+        ``z`` when ``inplace_output`` is set.  ``before_first_write`` is called once, right before
+        the first kernel that writes ``z`` is enqueued (see ``PairformerTrunk``)."""
         check_inference(z, "Pairformer block")
         if self.training:
             raise RuntimeError("The hip Pairformer block is inference-only (call .eval()).")
         _contiguous_io(z, "z")
-        _trimul_inplace(self.tri_mul_out, z, pair_mask)
+        _trimul_inplace(self.tri_mul_out, z, pair_mask, before_write=before_first_write)
         _trimul_inplace(self.tri_mul_in, z, pair_mask)
         _triattn_inplace(self.tri_att_start, z, pair_mask)
         _triattn_inplace(self.tri_att_end, z, pair_mask)
@@ -130,11 +133,19 @@ class PairSingleBlock(nn.Module):
         """z [B, N, N, Cz], s [B, N, Cs], pair_mask [B, N, N], mask [B, N]; s is updated in place."""
         _contiguous_io(s, "s")
         z = self.pair_block(z, pair_mask, inplace_output=inplace_output)
+        self.single_track(z, s, mask)
+        return z, s
+
+    def single_track(self, z: torch.Tensor, s: torch.Tensor, mask: torch.Tensor, after_bias=None) -> None:
+        """``s += SelfAttentionPairBias(s; bias(z))``, ``s += Transition_4(s)`` on the current stream.
+        ``after_bias`` is called once the last kernel that reads ``z`` has been enqueued."""
         B = z.shape[0]
         pb_params = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_pair_bias.weight)
         pb_blob = cached_blob(self, "_hip_pair_bias_cache", cache_key(pb_params, z, torch.bfloat16),
                               lambda: ops.pair_bias_pack(*pb_params, device=z.device))
         tiles = ops.pair_bias_project(z, pb_blob, self.num_heads, eps=self.layernorm_z.eps)
+        if after_bias is not None:
+            after_bias()
         att = self.attention
         check_inf(att)
         params = _parameters(att)
@@ -144,23 +155,65 @@ class PairSingleBlock(nn.Module):
         ops.apb_forward(s, None, tiles, mask.reshape(B, -1), blob, att.num_heads, 0, True, B > 1,
                         eps=norm_eps(att), residual=s, out=s)
         hip_transition(self.transition, s, residual=s, out=s)
-        return z, s
 
 
 class PairformerTrunk(nn.Module):
-    """A stack of ``PairSingleBlock``; z and s are updated in place block after block."""
+    """A stack of ``PairSingleBlock``; z and s are updated in place block after block.
+
+    With ``overlap_tracks`` (default) the single track of block b runs on a second HIP stream
+    while the pair track of block b+1 runs on the caller's stream: the single track only reads
+    the final ``z`` of its block (for the pair bias), and the next pair track never touches ``s``.
+    Events keep the reference's order of effects: the single track starts after its block's last
+    write of ``z``, and the next block's first write of ``z`` waits until the pair-bias kernel has
+    read it.  Both streams have the default priority.  The result is bit-identical to the serial
+    schedule."""
 
     def __init__(self, num_blocks: int, channel_s: int = 384, channel_z: int = 128,
-                 num_heads: int = 16, num_tri_heads: int = 4, kernel_backend: str = "hip"):
+                 num_heads: int = 16, num_tri_heads: int = 4, kernel_backend: str = "hip",
+                 overlap_tracks: bool = True):
         super().__init__()
+        self.overlap_tracks = overlap_tracks
         self.blocks = nn.ModuleList(
             PairSingleBlock(channel_s, channel_z, num_heads, num_tri_heads, kernel_backend)
             for _ in range(num_blocks))
+        self._side = {}
+
+    def _side_stream(self, device: torch.device) -> torch.cuda.Stream:
+        key = (device.type, device.index)
+        if key not in self._side:
+            self._side[key] = torch.cuda.Stream(device=device)
+        return self._side[key]
 
     def forward(self, z, s, pair_mask, mask):
-        for blk in self.blocks:
+        return run_blocks(list(self.blocks), z, s, pair_mask, mask,
+                          self._side_stream(z.device) if self.overlap_tracks and z.is_cuda else None)
+
+
+def run_blocks(blocks, z, s, pair_mask, mask, side: "torch.cuda.Stream | None" = None):
+    """Apply ``PairSingleBlock``s in turn to (z, s), in place.  With a ``side`` stream the single
+    tracks run there, overlapped with the following block's pair track (see ``PairformerTrunk``)."""
+    if side is None or len(blocks) == 0:
+        for blk in blocks:
             z, s = blk(z, s, pair_mask, mask, inplace_output=True)
         return z, s
+    _contiguous_io(s, "s")
+    main = torch.cuda.current_stream(z.device)
+    side.wait_stream(main)                     # s (and the weights) may have been produced on main
+    z_read = None                              # event: the previous block's pair-bias kernel has read z
+    for blk in blocks:
+        wait = None
+        if z_read is not None:
+            ev = z_read
+            wait = lambda ev=ev: main.wait_event(ev)
+        z = blk.pair_block(z, pair_mask, inplace_output=True, before_first_write=wait)
+        z_done = torch.cuda.Event()
+        z_done.record(main)
+        z_read = torch.cuda.Event()
+        with torch.cuda.stream(side):
+            side.wait_event(z_done)
+            blk.single_track(z, s, mask, after_bias=lambda ev=z_read: ev.record(side))
+    main.wait_stream(side)
+    return z, s
 
 
 class ParcaeStep(nn.Module):

@@ -78,8 +78,12 @@ def trimul_pack(ln_in_w, ln_in_b, p_in_w, g_in_w, ln_out_w, ln_out_b, p_out_w, g
 
 def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, direction: str,
                    eps: float = 1e-5, residual: torch.Tensor | None = None,
-                   out: torch.Tensor | None = None) -> torch.Tensor:
-    """``out = (residual or 0) + TriangleMultiplication(z, mask)`` for z [*, N, N, C]."""
+                   out: torch.Tensor | None = None, before_write=None) -> torch.Tensor:
+    """``out = (residual or 0) + TriangleMultiplication(z, mask)`` for z [*, N, N, C].
+
+    ``before_write``: called after the kernels that only read ``z`` have been enqueued and before
+    the one that writes ``out`` (which may be ``z``): the place to make this stream wait for
+    another stream's reads of ``z``."""
     dev = _require_cuda(z, mask, blob, residual, out)
     if direction not in ("outgoing", "incoming"):
         raise ValueError(f"unknown direction: {direction!r} (expected 'outgoing'/'incoming')")
@@ -101,13 +105,22 @@ def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, dire
     L = _lib.lib()
     ws_bytes = L.kfh_trimul_workspace_bytes(N, C)
     if ws_bytes == 0:
-        raise NotImplementedError(f"hip triangle multiplication is built for C=128, got {C}")
+        raise NotImplementedError(f"hip triangle multiplication is built for C=128 and C=256, got {C}")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    d = KFH_INCOMING if direction == "incoming" else KFH_OUTGOING
     with torch.cuda.device(dev):
-        check(L.kfh_trimul_forward(zc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
-                                   out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C,
-                                   KFH_INCOMING if direction == "incoming" else KFH_OUTGOING,
-                                   float(eps), _io_dtype(zc), _stream(dev)))
+        if before_write is None or B != 1:
+            if before_write is not None:
+                before_write()
+            check(L.kfh_trimul_forward(zc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
+                                       out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C, d,
+                                       float(eps), _io_dtype(zc), _stream(dev)))
+        else:
+            args = (zc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual), out.data_ptr(),
+                    ws.data_ptr(), ws_bytes, B, N, C, d, float(eps), _io_dtype(zc))
+            check(L.kfh_trimul_forward_stages(*args, _lib.KFH_STAGE_IN | _lib.KFH_STAGE_CORE, _stream(dev)))
+            before_write()
+            check(L.kfh_trimul_forward_stages(*args, _lib.KFH_STAGE_OUT, _stream(dev)))
     return out
 
 

@@ -151,6 +151,13 @@ def test_trunk_three_blocks():
     print(assert_stream_close(zg, zs, zw, "trunk z", max_flip_frac=2e-3, max_ulps=8), flush=True)
     print(assert_stream_close(sg, ss, sw, "trunk s", max_flip_frac=2e-3, max_ulps=8), flush=True)
     assert (zg.cpu()[~pm] == 0).all()
+    # the two-stream schedule (single track of block b beside the pair track of block b+1) gives
+    # the same bits as the serial one
+    from kfold_amd import modules as M
+    with torch.no_grad():
+        zs_, ss_ = M.run_blocks(list(hip.blocks), zb.to(DEV), sb.to(DEV), pm.to(DEV), tok.to(DEV), side=None)
+        torch.cuda.synchronize()
+    assert hip.overlap_tracks and torch.equal(zs_, zg) and torch.equal(ss_, sg)
     # the same three blocks with an fp32 stream: no storage rounding, unscaled limits end to end
     with torch.no_grad():
         zf, sf = hip(zb.float().to(DEV), sb.float().to(DEV), pm.to(DEV), tok.to(DEV))

@@ -233,6 +233,11 @@ def test_trunk_48_blocks_n1024():
         assert torch.isfinite(z48).all() and (z48[~pmd] == 0).all()
     zfull, sfull = run(48)
     assert torch.equal(zfull, z48) and torch.equal(sfull, s48), "run-to-run results differ"
+    # the trunk module's own schedule (single tracks on a second stream) gives the same bits
+    with torch.no_grad():
+        zt, st_ = hip(zb.to(DEV), sb.to(DEV), pmd, tokd)
+        torch.cuda.synchronize()
+    assert torch.equal(zt, z48) and torch.equal(st_, s48), "two-stream trunk differs from the serial one"
     print(f"  after 48 blocks: |z| max {z48.abs().max().item():.2f} rms "
           f"{z48.float().pow(2).mean().sqrt().item():.3f}", flush=True)
 
