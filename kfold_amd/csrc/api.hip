@@ -153,7 +153,7 @@ TaSizes ta_sizes(int N) {
     s.frag = align_up((size_t)N * 4 * s.nb * 2048);
     s.bias = align_up((size_t)4 * s.nb * s.nb * 2048);
     s.codes = align_up((size_t)N * s.nb * 32);
-    s.total = 5 * s.frag + s.bias + s.codes;
+    s.total = 4 * s.frag + s.bias + s.codes;
     return s;
 }
 }  // namespace
@@ -187,14 +187,14 @@ int kfh_triattn_pack(const void* ln_w, const void* ln_b, const void* q_w, const 
                            b + kTaProjOff + (2 * h) * kBlockBytes, stream);
         launch_pack_blocks(k_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, 1.f,
                            b + kTaProjOff + (2 * h + 1) * kBlockBytes, stream);
-        launch_pack_blocks(g_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, 1.f,
-                           b + kTaProjOff + (8 + 2 * h) * kBlockBytes, stream);
         launch_pack_blocks(v_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, 1.f,
-                           b + kTaProjOff + (8 + 2 * h + 1) * kBlockBytes, stream);
+                           b + kTaProjOff + (8 + h) * kBlockBytes, stream);
+        launch_pack_blocks(g_w, w_dtype, 32, C, C, 32 * h, 1, ROW_NATURAL, K_NATURAL, -kLog2e,
+                           b + kTaGateOff + h * kBlockBytes, stream);
     }
     launch_pack_blocks(bias_w, w_dtype, H, C, C, 0, 1, ROW_NATURAL, K_NATURAL, kLog2e,
-                       b + kTaProjOff + 16 * kBlockBytes, stream);
-    launch_fill_zero(b + kTaProjOff + 17 * kBlockBytes, kBlockBytes, stream);
+                       b + kTaProjOff + 12 * kBlockBytes, stream);
+    launch_fill_zero(b + kTaProjOff + 13 * kBlockBytes, kBlockBytes, stream);
     launch_pack_blocks(o_w, w_dtype, C, C, C, 0, 4, ROW_INTERLEAVE4, K_ACC, 1.f, b + kTaOutOff, stream);
     float* ln = reinterpret_cast<float*>(b + kTaLnOff);
     launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);
@@ -249,10 +249,9 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
         return fail(KFH_EINVAL, "triattn_forward: workspace %zu < %zu bytes", workspace_bytes, sz.total);
     char* w = static_cast<char*>(workspace);
     TriattnWorkspace ws;
-    ws.qf = w; ws.kf = w + sz.frag; ws.vf = w + 2 * sz.frag; ws.gf = w + 3 * sz.frag;
-    ws.of = w + 4 * sz.frag;
-    ws.biast = reinterpret_cast<uint16_t*>(w + 5 * sz.frag);
-    ws.codes = reinterpret_cast<uint8_t*>(w + 5 * sz.frag + sz.bias);
+    ws.qf = w; ws.kf = w + sz.frag; ws.vf = w + 2 * sz.frag; ws.of = w + 3 * sz.frag;
+    ws.biast = reinterpret_cast<uint16_t*>(w + 4 * sz.frag);
+    ws.codes = reinterpret_cast<uint8_t*>(w + 4 * sz.frag + sz.bias);
     const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
     for (int b = 0; b < B; ++b) {
         const size_t off = (size_t)b * N * N * C * esz;

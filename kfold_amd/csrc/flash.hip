@@ -411,11 +411,14 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
             }
         }
 
+        const bool gated = p.gf != nullptr;     // triangle attention gates in its output kernel
         u32x4 gg[2][2];
+        if (gated) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t) {
-            gg[t][0] = gf[row_units + qb[t] * 128 + lane];
-            gg[t][1] = gf[row_units + qb[t] * 128 + 64 + lane];
+            for (int t = 0; t < 2; ++t) {
+                gg[t][0] = gf[row_units + qb[t] * 128 + lane];
+                gg[t][1] = gf[row_units + qb[t] * 128 + 64 + lane];
+            }
         }
         if (a + a_step < p.nrows) request_row(a + a_step);
 #pragma unroll
@@ -423,14 +426,19 @@ __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashA
             if (t == 1 && !have_b) break;
             const float inv = fast_rcp(xhalf_sum(l[t]));
             const size_t u0 = row_units + qb[t] * 128 + lane;
-            const u32x4 g0 = gg[t][0], g1 = gg[t][1];
             f32x16 og;
+            if (gated) {
+                const u32x4 g0 = gg[t][0], g1 = gg[t][1];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                og[2 * e] = o[t][0][2 * e] * inv * bf16_lo(g0[e]);
-                og[2 * e + 1] = o[t][0][2 * e + 1] * inv * bf16_hi(g0[e]);
-                og[8 + 2 * e] = o[t][0][8 + 2 * e] * inv * bf16_lo(g1[e]);
-                og[8 + 2 * e + 1] = o[t][0][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
+                for (int e = 0; e < 4; ++e) {
+                    og[2 * e] = o[t][0][2 * e] * inv * bf16_lo(g0[e]);
+                    og[2 * e + 1] = o[t][0][2 * e + 1] * inv * bf16_hi(g0[e]);
+                    og[8 + 2 * e] = o[t][0][8 + 2 * e] * inv * bf16_lo(g1[e]);
+                    og[8 + 2 * e + 1] = o[t][0][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) og[v] = o[t][0][v] * inv;
             }
             bf16x8 f0, f1;
             acc_to_frags(og, f0, f1);
@@ -609,14 +617,19 @@ __global__ __launch_bounds__(512, (DKS == 2 ? (PERROW ? 3 : 4) : 2)) void flash_
 #pragma unroll
         for (int d = 0; d < DV; ++d) {
             const size_t u0 = qblk_units(a, qb) + (2 * d) * 64 + lane;
-            const u32x4 g0 = gf[u0], g1 = gf[u0 + 64];
             f32x16 og;
+            if (p.gf != nullptr) {
+                const u32x4 g0 = gf[u0], g1 = gf[u0 + 64];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                og[2 * e] = o[r][d][2 * e] * inv * bf16_lo(g0[e]);
-                og[2 * e + 1] = o[r][d][2 * e + 1] * inv * bf16_hi(g0[e]);
-                og[8 + 2 * e] = o[r][d][8 + 2 * e] * inv * bf16_lo(g1[e]);
-                og[8 + 2 * e + 1] = o[r][d][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
+                for (int e = 0; e < 4; ++e) {
+                    og[2 * e] = o[r][d][2 * e] * inv * bf16_lo(g0[e]);
+                    og[2 * e + 1] = o[r][d][2 * e + 1] * inv * bf16_hi(g0[e]);
+                    og[8 + 2 * e] = o[r][d][8 + 2 * e] * inv * bf16_lo(g1[e]);
+                    og[8 + 2 * e + 1] = o[r][d][8 + 2 * e + 1] * inv * bf16_hi(g1[e]);
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; ++v) og[v] = o[r][d][v] * inv;
             }
             bf16x8 f0, f1;
             acc_to_frags(og, f0, f1);

@@ -52,24 +52,26 @@ int launch_trimul_out_wide(const uint16_t* planes_y, const void* z, const char* 
 
 // ---- triangle attention (triattn.hip) ------------------------------------------------------
 // Packed weight blob of one triangle-attention module (C = 128, 4 heads x 32):
-//   [0, 144K)     9 steps x 2 blocks: {q_h,k_h} h=0..3, {g_h,v_h} h=0..3, {pair bias, zero};
+//   [0, 112K)     7 steps x 2 blocks: {q_h,k_h} h=0..3, {v_0,v_1}, {v_2,v_3}, {pair bias, zero};
 //                 q and the pair bias are pre-multiplied by log2(e) (and q by 1/sqrt(32))
+//   [112K, 144K)  gate g_h, 4 blocks, pre-multiplied by -log2(e) (output phase)
 //   [144K, 176K)  o projection, 4 blocks (ROW_INTERLEAVE4, K_ACC)
 //   [176K, +1K)   fp32: LN gamma, beta
 constexpr size_t kTaProjOff = 0;
+constexpr size_t kTaGateOff = 14 * kBlockBytes;
 constexpr size_t kTaOutOff = 18 * kBlockBytes;
 constexpr size_t kTaLnOff = 22 * kBlockBytes;
 constexpr size_t kTaBlobBytes = kTaLnOff + 2 * kC * sizeof(float);
 
 struct TriattnWorkspace {
-    void *qf, *kf, *vf, *gf, *of;   // fragment buffers, N * 4 * nb * 2 KiB each
+    void *qf, *kf, *vf, *of;        // fragment buffers, N * 4 * nb * 2 KiB each
     uint16_t* biast;                 // 4 * nb * nb bf16 tiles of 2 KiB
     uint8_t* codes;                  // N * nb * 32 key codes
 };
 
 // ---- attention core (flash.hip) --------------------------------------------------------------
 struct FlashArgs {
-    const void *qf, *kf, *vf, *gf;   // fragment-order operands
+    const void *qf, *kf, *vf, *gf;   // fragment-order operands; gf (the sigmoid gate) may be null
     void* of;                         // gated output fragments
     const void* biast;                // bf16 bias tiles [batch][h][query block][key block] (bias_tile_elem layout)
     const uint8_t* codes;             // [nrows][nb*32] key codes

@@ -9,9 +9,11 @@
 //     L[i,h,j,k] = q[i,j,h] . k[i,k,h] + beta[h,j,k] - 1e9 * (1 - mask'[i,k])
 //     o[i,j,h]   = softmax_k(L) v[i,k,h] ;  out'[i,j] = W_o (o[i,j] * sigmoid(g[i,j]))
 //
-// triattn_proj_kernel  x' rows -> LN -> q,k,v,gate in MFMA fragment order + bias tiles + key codes
+// triattn_proj_kernel  x' rows -> LN -> q,k,v in MFMA fragment order + bias tiles + key codes
 // flash_kernel         (flash.hip) per (row, head, 32 queries): online-softmax attention
-// triattn_out_kernel   gated o fragments -> W_o -> (+ residual) -> out (transposed back)
+// triattn_out_kernel   o fragments * sigmoid(W_g LN(x')) -> W_o -> (+ residual) -> out (transposed
+//                      back); the gate is recomputed from x' here (its rows are read for the
+//                      residual anyway) instead of being stored by the projection kernel
 //
 // Fragment buffers: [row a][head h][position block of 32][k-step 0..1][lane][8 bf16], the
 // accumulator-to-fragment order of common.hpp, so the three kernels exchange MFMA operands
@@ -39,8 +41,7 @@ template <int IO, int PB>
 __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kernel(
     const void* __restrict__ x, const uint8_t* __restrict__ mask, const char* __restrict__ blob,
     bf16x8* __restrict__ qf, bf16x8* __restrict__ kf, bf16x8* __restrict__ vf,
-    bf16x8* __restrict__ gf, uint16_t* __restrict__ biast, uint8_t* __restrict__ codes, int N, int nb,
-    int ending, float eps) {
+    uint16_t* __restrict__ biast, uint8_t* __restrict__ codes, int N, int nb, int ending, float eps) {
     __shared__ __attribute__((aligned(16))) char smem[kTileA * kXS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
@@ -85,10 +86,10 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
     }
     __syncthreads();
 
-    // 9 steps of two 32-column weight blocks (16 KiB), double-buffered in LDS:
-    //   0..3  { q_h , k_h }   both with channels as accumulator rows (weights = A operand)
-    //   4..7  { g_h , v_h }   g_h like q; v_h with positions as rows (activations = A operand)
-    //   8     { pair bias, - } rows 0..3 of the block are the 4 heads
+    // 7 steps of two 32-column weight blocks (16 KiB), double-buffered in LDS:
+    //   0..3  { q_h , k_h }      channels as accumulator rows (weights = A operand)
+    //   4, 5  { v_2s , v_2s+1 }  positions as rows (activations = A operand)
+    //   6     { pair bias, - }   rows 0..3 of the block are the 4 heads
     auto commit = [&](int s) {
 #pragma unroll
         for (int i = 0; i < NPRE; ++i)
@@ -106,10 +107,9 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
     commit(0);
     __syncthreads();
 
-    for (int s = 0; s < 8; ++s) {
+    for (int s = 0; s < 6; ++s) {
         prefetch(s + 1);
-        const bool gv = s >= 4;
-        const int h = s & 3;
+        const bool vv = s >= 4;
         f32x16 acc[2][PB];
 #pragma unroll
         for (int b = 0; b < 2; ++b)
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
             for (int pb = 0; pb < PB; ++pb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[b][pb][v] = 0.f;
-        if (!gv) {
+        if (!vv) {
 #pragma unroll
             for (int ks = 0; ks < kKS; ++ks) {
                 const bf16x8 w0 = wfrag(s, 0, ks), w1 = wfrag(s, 1, ks);
@@ -133,20 +133,21 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
                 const bf16x8 w0 = wfrag(s, 0, ks), w1 = wfrag(s, 1, ks);
 #pragma unroll
                 for (int pb = 0; pb < PB; ++pb) {
-                    acc[0][pb] = mfma32(w0, xf[pb][ks], acc[0][pb]);
+                    acc[0][pb] = mfma32(xf[pb][ks], w0, acc[0][pb]);
                     acc[1][pb] = mfma32(xf[pb][ks], w1, acc[1][pb]);
                 }
             }
-#pragma unroll
-            for (int pb = 0; pb < PB; ++pb)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[0][pb][v] = sigmoidf_fast(acc[0][pb][v]);
         }
 #pragma unroll
         for (int pb = 0; pb < PB; ++pb) {
             if (blk0 + pb < nb) {
-                store_frags(gv ? gf : qf, h, pb, acc[0][pb]);
-                store_frags(gv ? vf : kf, h, pb, acc[1][pb]);
+                if (!vv) {
+                    store_frags(qf, s, pb, acc[0][pb]);
+                    store_frags(kf, s, pb, acc[1][pb]);
+                } else {
+                    store_frags(vf, 2 * (s - 4), pb, acc[0][pb]);
+                    store_frags(vf, 2 * (s - 4) + 1, pb, acc[1][pb]);
+                }
             }
         }
         commit(s + 1);
@@ -164,7 +165,7 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
             for (int v = 0; v < 16; ++v) acc[pb][v] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < kKS; ++ks) {
-            const bf16x8 w0 = wfrag(8, 0, ks);
+            const bf16x8 w0 = wfrag(6, 0, ks);
 #pragma unroll
             for (int pb = 0; pb < PB; ++pb) acc[pb] = mfma32(w0, xf[pb][ks], acc[pb]);
         }
@@ -186,23 +187,66 @@ __global__ __launch_bounds__(512 / PB, (PB == 1 ? 4 : 2)) void triattn_proj_kern
 }
 
 // ------------------------------------------------------------------------------------------
-// output projection: out'[a][b] = W_o (gated o), 32 positions per wavefront, 8 wavefronts
+// output projection: out'[a][b] = W_o (o * sigmoid(W_g LN(x'[a][b]))), 32 positions per wavefront,
+// 8 wavefronts (model/primitives/triangle_attention.py:269-283)
 // ------------------------------------------------------------------------------------------
 template <int IO>
-__global__ __launch_bounds__(512, 3) void triattn_out_kernel(
-    const bf16x8* __restrict__ of, const char* __restrict__ blob, const void* residual, void* out,
-    int N, int nb, int ending) {
+__global__ __launch_bounds__(512, 2) void triattn_out_kernel(
+    const bf16x8* __restrict__ of, const void* x, const char* __restrict__ blob, const void* residual,
+    void* out, int N, int nb, int ending, float eps) {
+    __shared__ __attribute__((aligned(16))) char smem[kTileA * kXS];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
     const int a = blockIdx.y, t0 = blockIdx.x * kTileA;
     const int blk = (t0 >> 5) + wave;
+
+    // LN(x') rows of the tile -> LDS (every wavefront takes part, also one past the last block)
+    auto row_off = [&](int row) -> long long {
+        const int b = t0 + row;
+        if (b >= N) return -1;
+        const size_t pos = ending ? (size_t)b * N + a : (size_t)a * N + b;
+        return (long long)(pos * kC);
+    };
+    stage_ln_rows<IO, kTileA, decltype(row_off), 512>(
+        smem, x, reinterpret_cast<const float*>(blob + kTaLnOff), eps, tid, row_off);
+    __syncthreads();
     if (blk >= nb) return;
 
+    // (requesting the o fragments before the staging costs 6 more registers, which drops the
+    // kernel to one workgroup per CU: 172 instead of 122 us at N = 768)
     bf16x8 xf[kKS];
 #pragma unroll
     for (int h = 0; h < kH; ++h) {
         xf[2 * h] = of[frag_index(a, h, blk, 0, nb, lane)];
         xf[2 * h + 1] = of[frag_index(a, h, blk, 1, nb, lane)];
+    }
+    // gate of head h: channels as accumulator rows, so that the accumulator has the layout of
+    // the o fragments (k-step = register group of 8, see acc_to_frags); the weights are packed
+    // times -log2(e): sigmoid = 1 / (1 + exp2(acc))
+    {
+        bf16x8 zf[kKS];
+#pragma unroll
+        for (int ks = 0; ks < kKS; ++ks) zf[ks] = lds_frag(smem, wave * 32 + col, ks, half);
+        const bf16x8* wg = reinterpret_cast<const bf16x8*>(blob + kTaGateOff);
+#pragma unroll
+        for (int h = 0; h < kH; ++h) {
+            f32x16 g;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) g[v] = 0.f;
+#pragma unroll
+            for (int ks = 0; ks < kKS; ++ks) g = mfma32(wg[(h * kKS + ks) * 64 + lane], zf[ks], g);
+            const u32x4 o0 = __builtin_bit_cast(u32x4, xf[2 * h]), o1 = __builtin_bit_cast(u32x4, xf[2 * h + 1]);
+            f32x16 og;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                og[2 * e] = bf16_lo(o0[e]) * fast_rcp(1.0f + fast_exp2(g[2 * e]));
+                og[2 * e + 1] = bf16_hi(o0[e]) * fast_rcp(1.0f + fast_exp2(g[2 * e + 1]));
+                og[8 + 2 * e] = bf16_lo(o1[e]) * fast_rcp(1.0f + fast_exp2(g[8 + 2 * e]));
+                og[8 + 2 * e + 1] = bf16_hi(o1[e]) * fast_rcp(1.0f + fast_exp2(g[8 + 2 * e + 1]));
+            }
+            acc_to_frags(og, xf[2 * h], xf[2 * h + 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
     auto elem0 = [&](int v) -> size_t {
         const int b = min(blk * 32 + acc_row(v, half), N - 1);
@@ -273,20 +317,19 @@ int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char*
     bf16x8* qf = static_cast<bf16x8*>(ws.qf);
     bf16x8* kf = static_cast<bf16x8*>(ws.kf);
     bf16x8* vf = static_cast<bf16x8*>(ws.vf);
-    bf16x8* gf = static_cast<bf16x8*>(ws.gf);
     bf16x8* of = static_cast<bf16x8*>(ws.of);
     dim3 grid_rows((N + kTileA - 1) / kTileA, N), block(256);
     if (stages & KFH_STAGE_IN) {
         if (io_dtype == KFH_F32)
             hipLaunchKernelGGL((triattn_proj_kernel<KFH_F32, 1>), grid_rows, dim3(512), 0, stream, x, mask,
-                               blob, qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
+                               blob, qf, kf, vf, ws.biast, ws.codes, N, nb, ending, eps);
         else
             hipLaunchKernelGGL((triattn_proj_kernel<KFH_BF16, 1>), grid_rows, dim3(512), 0, stream, x, mask,
-                               blob, qf, kf, vf, gf, ws.biast, ws.codes, N, nb, ending, eps);
+                               blob, qf, kf, vf, ws.biast, ws.codes, N, nb, ending, eps);
     }
 
     FlashArgs fa{};
-    fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = gf; fa.of = of;
+    fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = nullptr; fa.of = of;
     fa.biast = ws.biast; fa.codes = ws.codes;
     fa.nrows = N; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
     if (stages & KFH_STAGE_CORE) {
@@ -296,11 +339,11 @@ int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char*
     if (!(stages & KFH_STAGE_OUT)) return 0;
 
     if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, dim3(512), 0, stream, of, blob,
-                           residual, out, N, nb, ending);
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, dim3(512), 0, stream, of, x, blob,
+                           residual, out, N, nb, ending, eps);
     else
-        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, dim3(512), 0, stream, of, blob,
-                           residual, out, N, nb, ending);
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, dim3(512), 0, stream, of, x, blob,
+                           residual, out, N, nb, ending, eps);
     return 0;
 }
 
