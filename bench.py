@@ -36,7 +36,7 @@ PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 CAL_COPY_BYTES = 256 << 20     # size of the counter-calibration copy
 # rocprofv3 FETCH_SIZE / WRITE_SIZE summary of this very command; bench.py only reads it
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hot_path_kernels_n768_hbm_traffic.md")
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "hot_path_kernels_n768_hbm_traffic.txt")
 
 
 def block_flops(n: int) -> dict:
@@ -571,7 +571,7 @@ def main() -> int:
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_BF16_TFLOPS, 4),
             "traffic": traffic_bytes,
-            "traffic_note": why_not or "FETCH_SIZE + WRITE_SIZE of profiles/hot_path_kernels_n768_hbm_traffic.md",
+            "traffic_note": why_not or "FETCH_SIZE + WRITE_SIZE of profiles/hot_path_kernels_n768_hbm_traffic.txt",
             "avg_launch_ms": round(flash_avg, 4),
             "flops_per_launch": flash_flops,
             "executed_flops": executed,

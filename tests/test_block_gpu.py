@@ -148,8 +148,8 @@ def test_trunk_three_blocks():
         zw, sw = ref(zb.float(), sb.float(), pm.float(), tok.float())
         zs, ss = stream(zb.float(), sb.float(), pm.float(), tok.float())
         zg, sg = hip(zb.to(DEV), sb.to(DEV), pm.to(DEV), tok.to(DEV))
-    print(assert_stream_close(zg, zs, zw, "trunk z", max_flip_frac=2e-3, max_ulps=8), flush=True)
-    print(assert_stream_close(sg, ss, sw, "trunk s", max_flip_frac=2e-3, max_ulps=8), flush=True)
+    print(assert_stream_close(zg, zs, zw, "trunk z", max_flip_frac=2e-3, n_adds=15), flush=True)
+    print(assert_stream_close(sg, ss, sw, "trunk s", max_flip_frac=2e-3, n_adds=6), flush=True)
     assert (zg.cpu()[~pm] == 0).all()
     # the two-stream schedule (single track of block b beside the pair track of block b+1) gives
     # the same bits as the serial one

@@ -48,7 +48,7 @@ def ulp_bf16(x: torch.Tensor) -> torch.Tensor:
     return torch.exp2(torch.floor(torch.log2(a)) - 7)
 
 
-def assert_stream_close(got, stream_ref, f32_ref, what="", max_flip_frac=2e-4, max_ulps=4.5):
+def assert_stream_close(got, stream_ref, f32_ref, what="", max_flip_frac=2e-4, n_adds=5):
     """A residual stream stored in bf16 (``got``) against the oracle run with the same bf16
     stream rounding (``stream_ref``) and the all-fp32 oracle (``f32_ref``).
 
@@ -56,8 +56,9 @@ def assert_stream_close(got, stream_ref, f32_ref, what="", max_flip_frac=2e-4, m
     * max-abs: an element of a bf16 stream moves in steps of its spacing (2^-6 for 2 <= |z| < 4,
       2^-5 above), so two correct implementations whose updates differ by far less than the
       limit still land on neighbouring bf16 values now and then ("rounding flips", a random
-      walk over the in-place adds).  Elements above the unscaled 2e-2 must be rare and within
-      a few bf16 steps;
+      walk over the ``n_adds`` in-place adds, one step at most per add).  Elements above the
+      unscaled 2e-2 must be rare and within ``n_adds`` bf16 steps of the reference value (plus
+      5e-3 for the difference of the updates themselves);
     * control: the distance to the fp32 oracle may not exceed, beyond a small margin, the
       distance of the bf16-stream oracle (exact fp32 arithmetic, same storage) to it — the
       error is then what bf16 storage of the stream costs, not kernel error."""
@@ -68,7 +69,7 @@ def assert_stream_close(got, stream_ref, f32_ref, what="", max_flip_frac=2e-4, m
     d = (g - s).abs()
     info = {"mean_abs_vs_stream": d.mean().item(), "max_abs_vs_stream": d.max().item(),
             "frac_above_2e-2": (d > MAX_ABS).float().mean().item(),
-            "max_ulps": (d / ulp_bf16(s)).max().item() if d.numel() else 0.0}
+            "max_steps_where_above": (d / ulp_bf16(s))[d > MAX_ABS].max().item() if (d > MAX_ABS).any() else 0.0}
     e_hip, e_str = errors(g, f), errors(s, f)
     info.update(hip_vs_f32=e_hip, stream_oracle_vs_f32=e_str)
     msg = f"{what}: {info}"
@@ -76,7 +77,7 @@ def assert_stream_close(got, stream_ref, f32_ref, what="", max_flip_frac=2e-4, m
     assert info["frac_above_2e-2"] <= max_flip_frac, msg
     big = d > MAX_ABS
     if big.any():
-        assert (d[big] / ulp_bf16(s[big])).max().item() <= max_ulps, msg
+        assert (d[big] <= n_adds * ulp_bf16(s[big]) + 5e-3).all(), msg
     assert e_hip["max_abs"] <= 1.25 * e_str["max_abs"] + 2e-3, msg
     assert e_hip["mean_abs"] <= 1.1 * e_str["mean_abs"] + 2e-4, msg
     return info
