@@ -122,3 +122,108 @@ def test_no_cpu_fallback_in_the_product_path():
             uses += 1
             assert current.startswith("cpu_baseline"), f"bench.py: oracle used in {current}()"
     assert uses >= 1
+
+
+def test_trunk_and_window_modules_keep_reference_names():
+    """State-dict keys of the trunk-level and local-window modules, spelled out from the reference's
+    attribute names (modules/tri_stack.py:31-151, model/model.py:201-217,
+    layers/folding/attention_pair_bias.py:161-204), and equal to the oracle's."""
+    from kfold_amd import layers, modules
+    from oracle import torch_path as O
+
+    pairs = [
+        (modules.TriangularBlock(256), O.TriangularBlock(256)),
+        (modules.TrianglularStack(256, 2), O.TrianglularStack(256, 2)),
+        (modules.ParcaeStep(128), O.ParcaeStep(128)),
+        (modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2), O.ParcaeTrunk(128, lm_blocks=1, main_blocks=2)),
+        (layers.CrossAttentionPairBias(128, 4, None), O.CrossAttentionPairBias(128, 4, None)),
+        (layers.CrossAttentionPairBias(128, 4, 64), O.CrossAttentionPairBias(128, 4, 64)),
+    ]
+    for hip, ref in pairs:
+        a, b = hip.state_dict(), ref.state_dict()
+        assert sorted(a) == sorted(b), type(hip).__name__
+        assert all(a[k].shape == b[k].shape for k in a), type(hip).__name__
+    blk = set(modules.TriangularBlock(256).state_dict())
+    assert {"tri_mul_out.linear_p_in.weight", "tri_mul_in.linear_g_out.weight",
+            "transition_z.swiglu.linear.weight", "transition_z.linear_out.weight"} <= blk
+    assert not any(k.startswith("tri_att") for k in blk)
+    trunk = set(modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2).state_dict())
+    assert {"parcae_log_a", "parcae_log_delta", "parcae_b_cont", "layernorm_z.weight",
+            "lm_stack.blocks.0.tri_mul_out.layernorm_in.weight",
+            "main_stack.blocks.1.transition_z.layernorm.weight"} <= trunk
+    win = set(layers.CrossAttentionPairBias(128, 4, 64).state_dict())
+    assert {"adaln_a_q.linear_g.weight", "adaln_a_k.linear_bias.weight", "linear_ada_out.bias",
+            "linear_q.bias", "linear_out.weight"} <= win and "linear_k.bias" not in win
+    plain = set(layers.CrossAttentionPairBias(128, 4, None).state_dict())
+    assert {"layernorm_a_q.weight", "layernorm_a_k.bias"} <= plain and "linear_ada_out.weight" not in plain
+
+
+def test_load_reference_weights_by_prefix():
+    """Loading goes by the reference's names below a prefix, ignores the rest of a checkpoint, and
+    refuses missing entries and wrong shapes."""
+    import torch
+
+    from kfold_amd import modules
+    from kfold_amd.runtime import load_reference_weights
+    from oracle import torch_path as O
+
+    torch.manual_seed(0)
+    ref = O.ParcaeTrunk(128, lm_blocks=1, main_blocks=2)
+    with torch.no_grad():
+        for p in ref.parameters():
+            p.copy_(torch.randn_like(p))
+    ckpt = {"trunk." + k: v for k, v in ref.state_dict().items()}
+    ckpt["distogram_head.weight"] = torch.zeros(3)               # something without a hip counterpart
+    hip = modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2)
+    used = load_reference_weights(hip, ckpt, prefix="trunk.")
+    assert sorted(used) == sorted(k for k in ckpt if k.startswith("trunk."))
+    for k, v in hip.state_dict().items():
+        assert torch.equal(v, ckpt["trunk." + k]), k
+    # one stack out of the same checkpoint
+    stack = modules.TrianglularStack(128, 2)
+    load_reference_weights(stack, ckpt, prefix="trunk.main_stack.")
+    assert torch.equal(stack.blocks[1].tri_mul_in.linear_p_in.weight,
+                       ckpt["trunk.main_stack.blocks.1.tri_mul_in.linear_p_in.weight"])
+    # a missing entry is an error unless strict is off; a wrong shape always is
+    short = dict(ckpt)
+    del short["trunk.parcae_log_a"]
+    with pytest.raises(KeyError, match="parcae_log_a"):
+        load_reference_weights(modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2), short, prefix="trunk.")
+    partial = modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2)
+    before = partial.parcae_log_a.detach().clone()
+    used = load_reference_weights(partial, short, prefix="trunk.", strict=False)
+    assert "trunk.parcae_log_a" not in used and torch.equal(partial.parcae_log_a, before)
+    bad = dict(ckpt)
+    bad["trunk.parcae_b_cont"] = torch.zeros(64, 64)
+    with pytest.raises(ValueError, match="parcae_b_cont"):
+        load_reference_weights(modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2), bad, prefix="trunk.")
+
+
+def test_recurrence_window_and_static_entry_points_check_arguments_without_gpu():
+    from kfold_amd import _lib
+
+    lib = _lib.lib()
+    assert lib.kfh_parcae_packed_bytes(128) > 0 and lib.kfh_parcae_packed_bytes(256) > lib.kfh_parcae_packed_bytes(128)
+    assert lib.kfh_parcae_packed_bytes(64) == 0 and lib.kfh_parcae_packed_bytes(384) == 0
+    rc = lib.kfh_parcae_step(None, None, None, None, None, 10, 64, 1e-5, 0, None)
+    assert rc == -2, lib.kfh_last_error()
+    rc = lib.kfh_parcae_step(None, None, None, None, None, 10, 128, 1e-5, 0, None)
+    assert rc == -1, lib.kfh_last_error()
+    # local attention windows: channels a multiple of 32, head dim at most 64
+    assert lib.kfh_cross_apb_packed_bytes(128, 4, 0) > 0 and lib.kfh_cross_apb_packed_bytes(128, 4, 64) > lib.kfh_cross_apb_packed_bytes(128, 4, 0)
+    assert lib.kfh_cross_apb_packed_bytes(128, 1, 0) == 0 and lib.kfh_cross_apb_packed_bytes(100, 4, 0) == 0
+    w1 = lib.kfh_cross_apb_workspace_bytes(10, 32, 128, 128, 4, 0)
+    w2 = lib.kfh_cross_apb_workspace_bytes(20, 32, 128, 128, 4, 0)
+    assert 0 < w1 < w2
+    # allocation-free transition: 8 MiB of static scratch; a request beyond it is refused before
+    # anything touches the GPU, with the limit in the message
+    cap = lib.kfh_transition_static_scratch_bytes()
+    assert cap == 8 << 20
+    rows_ok, rows_big = 2184, 2185
+    assert lib.kfh_transition_workspace_bytes(rows_ok, 384, 4) <= cap < lib.kfh_transition_workspace_bytes(rows_big, 384, 4)
+    rc = lib.kfh_transition_forward_static(None, None, None, None, None, rows_big, 384, 4, 1e-5, 0, None)
+    assert rc == -1 and b"static" in lib.kfh_last_error() and str(cap).encode() in lib.kfh_last_error()
+    rc = lib.kfh_transition_forward_static(None, None, None, None, None, -1, 384, 4, 1e-5, 0, None)
+    assert rc == -1
+    rc = lib.kfh_transition_forward_static(None, None, None, None, None, 10, 100, 4, 1e-5, 0, None)
+    assert rc == -2
