@@ -57,6 +57,40 @@ def _mask_bytes(mask: torch.Tensor, shape: torch.Size) -> torch.Tensor:
     return m.contiguous().view(torch.uint8)
 
 
+def _workspace(given: torch.Tensor | None, need: int, dev: torch.device) -> torch.Tensor:
+    """Scratch memory of a forward call: the caller's buffer if it passed one (reused across calls,
+    e.g. one buffer for all ops of a block that run on one stream), else a fresh allocation."""
+    if given is None:
+        return torch.empty(need, dtype=torch.uint8, device=dev)
+    if given.dtype != torch.uint8 or given.device != dev or not given.is_contiguous():
+        raise ValueError("workspace must be a contiguous uint8 tensor on the device of the inputs")
+    if given.numel() < need:
+        raise ValueError(f"workspace holds {given.numel()} bytes, this call needs {need}")
+    if given.data_ptr() % 256:
+        raise ValueError("workspace must be aligned to 256 bytes")
+    return given
+
+
+def workspace_bytes(op: str, **shape) -> int:
+    """Bytes of scratch memory a forward call needs (0: shape not supported): ``trimul`` (N, C),
+    ``triattn`` (N, C, heads), ``transition`` (rows, C, expansion), ``apb`` (S, L, C, heads,
+    cond_channels), ``cross_apb`` (W, Lq, Lk, C, heads, cond_channels).  Needs no GPU."""
+    L = _lib.lib()
+    g = shape.__getitem__
+    if op == "trimul":
+        return L.kfh_trimul_workspace_bytes(g("N"), g("C"))
+    if op == "triattn":
+        return L.kfh_triattn_workspace_bytes(g("N"), g("C"), g("heads"))
+    if op == "transition":
+        return L.kfh_transition_workspace_bytes(g("rows"), g("C"), g("expansion"))
+    if op == "apb":
+        return L.kfh_apb_workspace_bytes(g("S"), g("L"), g("C"), g("heads"), shape.get("cond_channels", 0))
+    if op == "cross_apb":
+        return L.kfh_cross_apb_workspace_bytes(g("W"), g("Lq"), g("Lk"), g("C"), g("heads"),
+                                               shape.get("cond_channels", 0))
+    raise ValueError(f"unknown op {op!r}")
+
+
 # ---------------------------------------------------------------------------------------
 # triangle multiplication
 # ---------------------------------------------------------------------------------------
@@ -78,8 +112,12 @@ def trimul_pack(ln_in_w, ln_in_b, p_in_w, g_in_w, ln_out_w, ln_out_b, p_out_w, g
 
 def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, direction: str,
                    eps: float = 1e-5, residual: torch.Tensor | None = None,
-                   out: torch.Tensor | None = None, before_write=None) -> torch.Tensor:
+                   out: torch.Tensor | None = None, before_write=None,
+                   workspace: torch.Tensor | None = None) -> torch.Tensor:
     """``out = (residual or 0) + TriangleMultiplication(z, mask)`` for z [*, N, N, C].
+
+    ``workspace``: optional uint8 scratch tensor of at least ``workspace_bytes("trimul", N=, C=)``
+    bytes to use instead of allocating one (its contents are overwritten).
 
     ``before_write``: called after the kernels that only read ``z`` have been enqueued and before
     the one that writes ``out`` (which may be ``z``): the place to make this stream wait for
@@ -106,7 +144,7 @@ def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, dire
     ws_bytes = L.kfh_trimul_workspace_bytes(N, C)
     if ws_bytes == 0:
         raise NotImplementedError(f"hip triangle multiplication is built for C=128 and C=256, got {C}")
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = _workspace(workspace, ws_bytes, dev)
     d = KFH_INCOMING if direction == "incoming" else KFH_OUTGOING
     with torch.cuda.device(dev):
         if before_write is None or B != 1:
@@ -143,8 +181,9 @@ def triattn_pack(ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w, device: torch.devi
 
 def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tensor, heads: int,
                     starting: bool, eps: float = 1e-5, residual: torch.Tensor | None = None,
-                    out: torch.Tensor | None = None) -> torch.Tensor:
-    """``out = (residual or 0) + TriangleAttention(x, mask)`` for x [*, N, N, C]."""
+                    out: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """``out = (residual or 0) + TriangleAttention(x, mask)`` for x [*, N, N, C]; ``workspace`` as in
+    ``trimul_forward`` (``workspace_bytes("triattn", N=, C=, heads=)``)."""
     dev = _require_cuda(x, mask, blob, residual, out)
     N, C = x.shape[-2], x.shape[-1]
     if x.dim() < 3 or x.shape[-3] != N:
@@ -169,7 +208,7 @@ def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tens
     if ws_bytes == 0:
         raise NotImplementedError(
             f"hip triangle attention is built for C=128, H=4, N<=8192; got C={C}, H={heads}, N={N}")
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = _workspace(workspace, ws_bytes, dev)
     with torch.cuda.device(dev):
         check(L.kfh_triattn_forward(xc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
                                     out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C, heads,
@@ -197,8 +236,9 @@ def transition_pack(ln_w, ln_b, swiglu_w, out_w, device: torch.device) -> torch.
 
 def transition_forward(x: torch.Tensor, blob: torch.Tensor, expansion: int, eps: float = 1e-5,
                        residual: torch.Tensor | None = None, mask: torch.Tensor | None = None,
-                       out: torch.Tensor | None = None) -> torch.Tensor:
-    """``out = ((residual or 0) + Transition(x)) * (mask or 1)`` over the last dim of x."""
+                       out: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """``out = ((residual or 0) + Transition(x)) * (mask or 1)`` over the last dim of x; ``workspace``
+    as in ``trimul_forward`` (``workspace_bytes("transition", rows=, C=, expansion=)``)."""
     dev = _require_cuda(x, blob, residual, mask, out)
     C = x.shape[-1]
     rows = x.numel() // C if x.numel() else 0
@@ -215,7 +255,7 @@ def transition_forward(x: torch.Tensor, blob: torch.Tensor, expansion: int, eps:
         return out
     L = _lib.lib()
     ws_bytes = L.kfh_transition_workspace_bytes(rows, C, expansion)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    ws = _workspace(workspace, ws_bytes, dev) if ws_bytes else None
     with torch.cuda.device(dev):
         check(L.kfh_transition_forward(xc.data_ptr(), blob.data_ptr(), _ptr(residual), _ptr(m8),
                                        out.data_ptr(), _ptr(ws), ws_bytes, rows, C, expansion,
@@ -290,8 +330,9 @@ def apb_pack(C: int, H: int, Cs: int, *, ln_w=None, ln_b=None, q_w, q_b, k_w, v_
 def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tensor, mask: torch.Tensor,
                 blob: torch.Tensor, heads: int, cond_channels: int, apply_norm: bool,
                 bias_per_sample: bool, eps: float = 1e-5, residual: torch.Tensor | None = None,
-                out: torch.Tensor | None = None) -> torch.Tensor:
-    """a [S, L, C]; s_cond [S or 1, L, Cs] or None; mask [S or 1, L]; tiles from the calls above."""
+                out: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """a [S, L, C]; s_cond [S or 1, L, Cs] or None; mask [S or 1, L]; tiles from the calls above;
+    ``workspace`` as in ``trimul_forward`` (``workspace_bytes("apb", S=, L=, C=, heads=, cond_channels=)``)."""
     dev = _require_cuda(a, s_cond, tiles, mask, blob, residual, out)
     S, Lq, C = a.shape
     ac = a.contiguous()
@@ -316,7 +357,7 @@ def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tenso
     ws_bytes = L.kfh_apb_workspace_bytes(S, Lq, C, heads, cond_channels)
     if ws_bytes == 0:
         raise NotImplementedError(f"hip pair-bias attention: unsupported shape S={S} L={Lq} C={C} H={heads}")
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = _workspace(workspace, ws_bytes, dev)
     with torch.cuda.device(dev):
         check(L.kfh_apb_forward(ac.data_ptr(), _ptr(sc), tiles.data_ptr(), m8.data_ptr(), blob.data_ptr(),
                                 _ptr(residual), out.data_ptr(), ws.data_ptr(), ws_bytes, S, Lq, C, heads,
@@ -390,8 +431,10 @@ def cross_apb_pack(C: int, H: int, Cs: int, device: torch.device, **weights) -> 
 
 def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias: torch.Tensor, mask: torch.Tensor,
                       blob: torch.Tensor, heads: int, cond_channels: int, eps: float = 1e-5,
-                      residual: torch.Tensor | None = None, out: torch.Tensor | None = None) -> torch.Tensor:
-    """a_q [W, Lq, C], a_k [W, Lk, C], s_q / s_k [W, L., Cs] or None, pair_bias [W, H, Lq, Lk], mask [W, Lk]."""
+                      residual: torch.Tensor | None = None, out: torch.Tensor | None = None,
+                      workspace: torch.Tensor | None = None) -> torch.Tensor:
+    """a_q [W, Lq, C], a_k [W, Lk, C], s_q / s_k [W, L., Cs] or None, pair_bias [W, H, Lq, Lk], mask [W, Lk];
+    ``workspace`` as in ``trimul_forward`` (``workspace_bytes("cross_apb", W=, Lq=, Lk=, C=, heads=, cond_channels=)``)."""
     dev = _require_cuda(a_q, a_k, s_q, s_k, pair_bias, mask, blob, residual, out)
     W, Lq, C = a_q.shape
     Lk = a_k.shape[1]
@@ -418,7 +461,7 @@ def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias:
     ws_bytes = L.kfh_cross_apb_workspace_bytes(W, Lq, Lk, C, heads, cond_channels)
     if ws_bytes == 0:
         raise NotImplementedError(f"hip cross attention: unsupported shape W={W} Lq={Lq} Lk={Lk} C={C} H={heads}")
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    ws = _workspace(workspace, ws_bytes, dev)
     with torch.cuda.device(dev):
         check(L.kfh_cross_apb_forward(aq.data_ptr(), ak.data_ptr(), _ptr(sq), _ptr(sk), pb.data_ptr(),
                                       _io_dtype(pb), m8.data_ptr(), blob.data_ptr(), _ptr(residual),

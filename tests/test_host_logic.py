@@ -1,0 +1,278 @@
+"""Host-side plumbing of the hip backend, run without a GPU.
+
+The library handle is replaced by a recorder that checks every call against the ctypes signature
+table (argument count and types), answers the size queries with the real library (they need no
+GPU) and records the converted arguments instead of launching anything.  What is checked here is
+what the Python layer decides: which entry points run in which order, which tensors alias, which
+flags, sizes and eps values are passed, when weights are repacked.  Nothing is computed, so these
+tests say nothing about numerics; the GPU tests do."""
+
+import contextlib
+import sys
+
+import pytest
+import torch
+
+
+class Recorder:
+    def __init__(self, real, signatures):
+        self.real, self.signatures, self.calls = real, signatures, []
+
+    def __getattr__(self, name):
+        res, argtypes = self.signatures[name]              # KeyError: not in the header
+        if name.endswith("_bytes") or name in ("kfh_version", "kfh_last_error"):
+            return getattr(self.real, name)
+
+        def call(*args):
+            assert len(args) == len(argtypes), f"{name}: {len(args)} arguments, header has {len(argtypes)}"
+            conv = tuple(None if a is None else t(a).value for a, t in zip(args, argtypes))
+            self.calls.append((name, conv))
+            return 0
+        return call
+
+    def names(self, suffixes=("_forward", "_forward_stages", "_project", "_step", "_from_dense")):
+        return [n for n, _ in self.calls if n.endswith(suffixes)]
+
+    def of(self, name):
+        return [a for n, a in self.calls if n == name]
+
+
+@pytest.fixture
+def rec(monkeypatch):
+    from kfold_amd import _lib, layers, modules, ops, primitives  # noqa: F401  (patched below)
+
+    r = Recorder(_lib.lib(), _lib.SIGNATURES)
+    monkeypatch.setattr(_lib, "lib", lambda: r)
+
+    def any_device(*tensors):
+        for t in tensors:
+            if t is not None:
+                return t.device
+    monkeypatch.setattr(ops, "_require_cuda", any_device)
+    monkeypatch.setattr(ops, "_stream", lambda dev: 0)
+    monkeypatch.setattr(torch.cuda, "device", lambda dev: contextlib.nullcontext())
+
+    def grad_only(x, what):
+        if torch.is_grad_enabled():
+            raise RuntimeError(f"The hip {what} backend is inference-only.")
+    for name, mod in list(sys.modules.items()):
+        if name.startswith("kfold_amd") and hasattr(mod, "check_inference"):
+            monkeypatch.setattr(mod, "check_inference", grad_only)
+    return r
+
+
+def _inside(ptr, t):
+    return t.data_ptr() <= ptr < t.data_ptr() + max(t.numel() * t.element_size(), 1)
+
+
+def test_pair_single_block_call_sequence_and_aliasing(rec):
+    from kfold_amd import modules, ops
+
+    N = 8
+    blk = modules.PairSingleBlock().eval()
+    blk.pair_block.tri_mul_in.layernorm_in.eps = 3e-5
+    blk.pair_block.tri_att_end.layer_norm.eps = 7e-6
+    z = torch.zeros(1, N, N, 128, dtype=torch.bfloat16)
+    s = torch.zeros(1, N, 384, dtype=torch.bfloat16)
+    tok = torch.ones(1, N, dtype=torch.bool)
+    tok[:, -2:] = False
+    pair = tok[:, :, None] & tok[:, None, :]
+    with torch.no_grad():
+        z_out, s_out = blk(z, s, pair, tok, inplace_output=True)
+    assert z_out.data_ptr() == z.data_ptr() and s_out.data_ptr() == s.data_ptr()
+    assert rec.names() == ["kfh_trimul_forward", "kfh_trimul_forward", "kfh_triattn_forward",
+                           "kfh_triattn_forward", "kfh_transition_forward", "kfh_pair_bias_project",
+                           "kfh_apb_forward", "kfh_transition_forward"]
+    out_call, in_call = rec.of("kfh_trimul_forward")
+    for c, direction, eps in ((out_call, 0, 1e-5), (in_call, 1, 3e-5)):
+        x, mask, blob, resid, out, ws, ws_bytes, B, n, C, d, e, io, stream = c
+        assert x == resid == out == z.data_ptr(), "tri-mul runs in place on z with the residual fused"
+        assert (B, n, C, d, io) == (1, N, 128, direction, 0)
+        assert e == pytest.approx(eps)
+        assert ws_bytes == ops.workspace_bytes("trimul", N=N, C=128) and ws
+    start, end = rec.of("kfh_triattn_forward")
+    assert start[11] == 0 and end[11] == 1, "starting node first, then the ending node"
+    assert start[12] == pytest.approx(1e-5) and end[12] == pytest.approx(7e-6)
+    assert start[0] == start[3] == start[4] == z.data_ptr()
+    pair_tr, single_tr = rec.of("kfh_transition_forward")
+    assert pair_tr[0] == pair_tr[2] == pair_tr[4] == z.data_ptr() and pair_tr[3], "final mask fused"
+    assert (pair_tr[7], pair_tr[8], pair_tr[9]) == (N * N, 128, 2)
+    assert single_tr[0] == single_tr[2] == single_tr[4] == s.data_ptr() and single_tr[3] is None
+    assert (single_tr[7], single_tr[8], single_tr[9]) == (N, 384, 4)
+    apb = rec.of("kfh_apb_forward")[0]
+    assert apb[0] == apb[5] == apb[6] == s.data_ptr() and apb[1] is None
+    assert apb[9:14] == (1, N, 384, 16, 0)
+    # the mask bytes handed to the kernels hold the pair mask
+    packs = [n for n, _ in rec.calls if n.endswith("_pack")]
+    assert sorted(packs) == sorted(["kfh_trimul_pack"] * 2 + ["kfh_triattn_pack"] * 2 + ["kfh_transition_pack"] * 2
+                                   + ["kfh_pair_bias_pack", "kfh_apb_pack"])
+
+
+def test_packed_weights_are_cached_until_a_parameter_changes(rec):
+    from kfold_amd import primitives
+
+    mod = primitives.TriangleMultiplicationOutgoing(128).eval()
+    x = torch.zeros(1, 4, 4, 128, dtype=torch.bfloat16)
+    m = torch.ones(1, 4, 4, dtype=torch.bool)
+    with torch.no_grad():
+        mod(x, m)
+        mod(x, m)
+        assert len(rec.of("kfh_trimul_pack")) == 1 and len(rec.of("kfh_trimul_forward")) == 2
+        mod.linear_p_out.weight.add_(1.0)                      # in-place update bumps the version
+        mod(x, m)
+        assert len(rec.of("kfh_trimul_pack")) == 2
+        mod.load_state_dict({k: v.clone() for k, v in mod.state_dict().items()})
+        mod(x, m)
+        assert len(rec.of("kfh_trimul_pack")) == 3
+    # module-level forward is out of place: z is read, a new tensor is written, no residual
+    c = rec.of("kfh_trimul_forward")[-1]
+    assert c[0] == x.data_ptr() and c[3] is None and c[4] != x.data_ptr()
+
+
+def test_caller_workspace_is_used_and_checked(rec):
+    from kfold_amd import ops
+
+    N = 8
+    z = torch.zeros(1, N, N, 128, dtype=torch.bfloat16)
+    m = torch.ones(1, N, N, dtype=torch.bool)
+    need_tm = ops.workspace_bytes("trimul", N=N, C=128)
+    need_ta = ops.workspace_bytes("triattn", N=N, C=128, heads=4)
+    assert need_tm > 0 and need_ta > 0
+    assert ops.workspace_bytes("trimul", N=N, C=64) == 0
+    with pytest.raises(ValueError):
+        ops.workspace_bytes("softmax", N=N)
+    blob = torch.zeros(16, dtype=torch.uint8)
+    base = torch.zeros(max(need_tm, need_ta) + 512, dtype=torch.uint8)
+    off = (-base.data_ptr()) % 256
+    ws = base[off:off + max(need_tm, need_ta)]
+    ops.trimul_forward(z, m, blob, "outgoing", workspace=ws)
+    ops.triattn_forward(z, m, blob, 4, True, workspace=ws)
+    assert rec.of("kfh_trimul_forward")[0][5] == ws.data_ptr()
+    assert rec.of("kfh_triattn_forward")[0][5] == ws.data_ptr()
+    assert rec.of("kfh_trimul_forward")[0][6] == need_tm and rec.of("kfh_triattn_forward")[0][6] == need_ta
+    with pytest.raises(ValueError, match="needs"):
+        ops.trimul_forward(z, m, blob, "outgoing", workspace=ws[:need_tm - 256])
+    with pytest.raises(ValueError, match="aligned"):
+        ops.trimul_forward(z, m, blob, "outgoing", workspace=base[off + 16:off + 16 + need_tm])
+    with pytest.raises(ValueError, match="uint8"):
+        ops.trimul_forward(z, m, blob, "outgoing", workspace=torch.zeros(need_tm, dtype=torch.int8))
+    # without one, each call allocates its own
+    ops.trimul_forward(z, m, blob, "incoming")
+    assert rec.of("kfh_trimul_forward")[-1][5] not in (None, ws.data_ptr())
+
+
+def test_wrappers_refuse_inconsistent_arguments_before_any_call(rec):
+    from kfold_amd import ops
+
+    z = torch.zeros(1, 8, 8, 128, dtype=torch.bfloat16)
+    m = torch.ones(1, 8, 8, dtype=torch.bool)
+    blob = torch.zeros(16, dtype=torch.uint8)
+    with pytest.raises(ValueError, match="direction"):
+        ops.trimul_forward(z, m, blob, "sideways")
+    with pytest.raises(ValueError, match=r"\[\*, N, N, C\]"):
+        ops.trimul_forward(z[:, :4], m[:, :4], blob, "outgoing")
+    with pytest.raises(ValueError, match="out must"):
+        ops.trimul_forward(z, m, blob, "outgoing", out=torch.zeros(1, 8, 8, 128))
+    with pytest.raises(ValueError, match="residual must"):
+        ops.triattn_forward(z, m, blob, 4, True, residual=z.float())
+    with pytest.raises(NotImplementedError):
+        ops.trimul_forward(torch.zeros(1, 8, 8, 64, dtype=torch.bfloat16), m, blob, "outgoing")
+    with pytest.raises(TypeError, match="bfloat16 and float32"):
+        ops.trimul_forward(z.half(), m, blob, "outgoing")
+    assert rec.names() == []
+    # an empty batch returns without a call
+    out = ops.trimul_forward(z[:0], m[:0], blob, "outgoing")
+    assert out.shape == (0, 8, 8, 128) and rec.names() == []
+
+
+def test_recurrent_trunk_call_sequence(rec):
+    """lm_stack -> recurrence step with the input sum fused -> main_stack, once per recycle
+    (reference: model/model.py:522-529)."""
+    from kfold_amd import modules
+
+    N = 8
+    trunk = modules.ParcaeTrunk(128, lm_blocks=1, main_blocks=2).eval()
+    z = torch.zeros(1, N, N, 128, dtype=torch.bfloat16)
+    z_in = torch.zeros_like(z)
+    z_lm = torch.zeros_like(z)
+    pair = torch.ones(1, N, N, dtype=torch.bool)
+    with torch.no_grad():
+        out = trunk(z, z_in, z_lm, pair, num_recycles=1)
+    assert out.data_ptr() == z.data_ptr()
+    block = ["kfh_trimul_forward", "kfh_trimul_forward", "kfh_transition_forward"]
+    recycle = block + ["kfh_parcae_step"] + block * 2
+    assert rec.names() == recycle * 2
+    for step in rec.of("kfh_parcae_step"):
+        zp, u, u_add, blob, outp, rows, C, eps, io, stream = step
+        assert zp == outp == z.data_ptr() and u_add == z_in.data_ptr()
+        assert u not in (z.data_ptr(), z_lm.data_ptr(), z_in.data_ptr()), "the LM stack works on a copy"
+        assert (rows, C, io) == (N * N, 128, 0)
+    # the triangular block's transition has expansion 4 and no mask; the state stays in place
+    tr = rec.of("kfh_transition_forward")
+    assert all(c[9] == 4 and c[3] is None for c in tr)
+    assert [c[0] == z.data_ptr() for c in tr] == [False, True, True] * 2
+    assert len(rec.of("kfh_parcae_pack")) == 1 and len(rec.of("kfh_trimul_pack")) == 6
+
+
+def test_serial_trunk_runs_blocks_in_order_on_the_same_tensors(rec):
+    from kfold_amd import modules
+
+    N = 8
+    trunk = modules.PairformerTrunk(2, overlap_tracks=False).eval()
+    z = torch.zeros(1, N, N, 128, dtype=torch.bfloat16)
+    s = torch.zeros(1, N, 384, dtype=torch.bfloat16)
+    tok = torch.ones(1, N, dtype=torch.bool)
+    pair = tok[:, :, None] & tok[:, None, :]
+    with torch.no_grad():
+        z_out, s_out = trunk(z, s, pair, tok)
+    assert z_out.data_ptr() == z.data_ptr() and s_out.data_ptr() == s.data_ptr()
+    one = ["kfh_trimul_forward", "kfh_trimul_forward", "kfh_triattn_forward", "kfh_triattn_forward",
+           "kfh_transition_forward", "kfh_pair_bias_project", "kfh_apb_forward", "kfh_transition_forward"]
+    assert rec.names() == one * 2
+    blobs = [c[2] for c in rec.of("kfh_trimul_forward")]
+    assert len(set(blobs)) == 4, "each block's two tri-mul modules have their own packed weights"
+
+
+def test_window_attention_flattens_leading_dimensions(rec):
+    """[B, W, L, C] windows go to the library as B*W windows; the conditioned variant passes both
+    conditioning tensors and the plain one none (reference:
+    layers/folding/attention_pair_bias.py:206-260)."""
+    from kfold_amd import layers
+
+    B, W, Lq, Lk, C, H, Cs = 2, 3, 32, 128, 128, 4, 64
+    a_q = torch.zeros(B, W, Lq, C, dtype=torch.bfloat16)
+    a_k = torch.zeros(B, W, Lk, C, dtype=torch.bfloat16)
+    bias = torch.zeros(B, W, H, Lq, Lk, dtype=torch.bfloat16)
+    mask = torch.ones(B, W, Lk, dtype=torch.bool)
+    with torch.no_grad():
+        plain = layers.CrossAttentionPairBias(C, H, None).eval()
+        out = plain(a_q, a_k, None, None, bias, mask)
+        assert out.shape == a_q.shape and out.dtype == a_q.dtype
+        cond = layers.CrossAttentionPairBias(C, H, Cs).eval()
+        s_q = torch.zeros(B, W, Lq, Cs, dtype=torch.bfloat16)
+        s_k = torch.zeros(B, W, Lk, Cs, dtype=torch.bfloat16)
+        cond(a_q, a_k, s_q, s_k, bias, mask)
+        with pytest.raises(AssertionError):
+            cond(a_q, a_k, None, None, bias, mask)
+    c0, c1 = rec.of("kfh_cross_apb_forward")
+    assert c0[12:18] == (B * W, Lq, Lk, C, H, 0) and c0[2] is None and c0[3] is None
+    assert c1[12:18] == (B * W, Lq, Lk, C, H, Cs) and c1[2] and c1[3]
+    assert c0[8] is None, "the module's forward returns the update without a residual"
+    assert c0[5] == 0, "bf16 pair bias is passed as it is"
+
+
+def test_other_widths_take_the_generic_entry_points(rec):
+    """Triangle multiplication at C=256 and triangle attention at C=64 (4 heads of 16) go through
+    the same entry points; unsupported widths are refused by the size queries."""
+    from kfold_amd import primitives
+
+    m = torch.ones(2, 8, 8, dtype=torch.bool)
+    with torch.no_grad():
+        primitives.TriangleMultiplicationIncoming(256).eval()(torch.zeros(2, 8, 8, 256, dtype=torch.bfloat16), m)
+        primitives.TriangleAttentionEndingNode(64, 4).eval()(torch.zeros(2, 8, 8, 64, dtype=torch.bfloat16), m)
+        with pytest.raises(NotImplementedError):
+            primitives.TriangleMultiplicationIncoming(64).eval()(torch.zeros(2, 8, 8, 64, dtype=torch.bfloat16), m)
+    tm = rec.of("kfh_trimul_forward")[0]
+    assert tm[7:11] == (2, 8, 256, 1)
+    ta = rec.of("kfh_triattn_forward")[0]
+    assert ta[7:12] == (2, 8, 64, 4, 1)

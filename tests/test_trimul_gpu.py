@@ -111,3 +111,30 @@ def test_trimul_weight_cache_invalidation_and_errors():
             hip(zd, md)
     with torch.no_grad(), pytest.raises(RuntimeError):
         hip(z.to(torch.bfloat16), pm)                # CPU tensor
+
+
+def test_caller_workspace_shared_by_consecutive_ops():
+    """One scratch buffer passed to triangle multiplication and triangle attention in turn (its
+    contents are whatever the previous op left) gives the results of per-call allocations."""
+    from kfold_amd import ops
+    from kfold_amd import primitives as P
+
+    print("case caller workspace shared by tri-mul and tri-attn", flush=True)
+    n = 72
+    tm = P.TriangleMultiplicationIncoming(128).eval()
+    ta = P.TriangleAttentionStartingNode(128, 4).eval()
+    synthetic.init_weights_(tm, 1)
+    synthetic.init_weights_(ta, 2)
+    tm, ta = tm.to(DEV), ta.to(DEV)
+    z, _, pm = synthetic.pair_inputs(n, 128, 9, seed=4)
+    zd, md = z.to(torch.bfloat16).to(DEV), pm.to(DEV)
+    with torch.no_grad():
+        want_tm, want_ta = tm(zd, md), ta(zd, md)            # packs the weights, allocates per call
+        need = max(ops.workspace_bytes("trimul", N=n, C=128), ops.workspace_bytes("triattn", N=n, C=128, heads=4))
+        ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)
+        for _ in range(2):
+            got_tm = ops.trimul_forward(zd, md, tm._hip_multiplication_cache, "incoming", workspace=ws)
+            got_ta = ops.triattn_forward(zd, md, ta._hip_attention_cache, 4, True, workspace=ws)
+            assert torch.equal(got_tm, want_tm) and torch.equal(got_ta, want_ta)
+        with pytest.raises(ValueError, match="needs"):
+            ops.trimul_forward(zd, md, tm._hip_multiplication_cache, "incoming", workspace=ws[:1024])
