@@ -293,3 +293,105 @@ def test_cross_apb_windows_vs_brute():
     want0 = brute.attention_pair_bias(qn[0].detach().numpy(), kn[0].detach().numpy(), bias[0].numpy(),
                                       mask[0].numpy(), pc, heads=2)
     assert np.allclose(core[0].detach().numpy(), want0, atol=1e-9)
+
+
+# ------------------------------------------------------------- trunk-level composition
+def _zero_linear_weights(module):
+    """All projections to zero: every update of a triangular block is then exactly zero."""
+    with torch.no_grad():
+        for name, p in module.named_parameters():
+            if p.dim() >= 2:
+                p.zero_()
+
+
+def test_triangular_block_and_stack_wiring():
+    """tri-mul out, tri-mul in, transition x4 recomposed from the individually pinned pieces; in
+    place, no triangle attention, no final mask (modules/tri_stack.py:138-150)."""
+    c, n = 4, 5
+    blk = _rand_init(O.TriangularBlock(c), 60, std=0.3)
+    assert blk.transition_z.swiglu.linear.weight.shape == (2 * 4 * c, c)
+    assert not hasattr(blk, "tri_att_start")
+    z = _rand((1, n, n, c), 61)
+    tok = torch.tensor([[True, True, True, True, False]])
+    pm = (tok[:, :, None] & tok[:, None, :]).double()
+    zz = z.clone()
+    zz = zz + blk.tri_mul_out(zz, pm)
+    zz = zz + blk.tri_mul_in(zz, pm)
+    zz = zz + blk.transition_z(zz)
+    z_in = z.clone()
+    out = blk(z_in, pm)
+    assert out is z_in and torch.allclose(out, zz, atol=1e-10)
+    assert out[0, -1, -1].abs().max() > 1e-3, "masked positions are not zeroed by this block"
+    # the order of the two directions matters, so a swap would show
+    sw = z.clone()
+    sw = sw + blk.tri_mul_in(sw, pm)
+    sw = sw + blk.tri_mul_out(sw, pm)
+    sw = sw + blk.transition_z(sw)
+    assert not torch.allclose(sw, zz, atol=1e-6)
+    stack = _rand_init(O.TrianglularStack(c, 3), 62, std=0.3)
+    want = z.clone()
+    for b in stack.blocks:
+        want = b(want.clone(), pm)
+    assert torch.allclose(stack(z.clone(), pm), want, atol=1e-10)
+
+
+def test_recurrent_trunk_wiring_and_closed_form():
+    """model/model.py:522-529: u = z_inputs + lm_stack(z_lm); z = a z + B LN(u); z = main_stack(z)."""
+    c, n = 4, 3
+    trunk = _rand_init(O.ParcaeTrunk(c, lm_blocks=1, main_blocks=2), 70, std=0.3)
+    g = torch.Generator().manual_seed(71)
+    with torch.no_grad():
+        trunk.parcae_log_a.copy_(0.5 * torch.randn(c, generator=g))
+        trunk.parcae_log_delta.copy_(torch.randn(c, generator=g))
+    z0, z_inputs, z_lm = _rand((1, n, n, c), 72), _rand((1, n, n, c), 73), _rand((1, n, n, c), 74)
+    pm = torch.ones(1, n, n, dtype=torch.float64)
+    step = O.ParcaeStep(c).double()
+    step.load_state_dict({k: v for k, v in trunk.state_dict().items() if "stack" not in k})
+    z = z0.clone()
+    for _ in range(2):
+        u = z_inputs + trunk.lm_stack(z_lm.clone(), pm)
+        z = step(z, u)
+        z = trunk.main_stack(z, pm)
+    lm_before = z_lm.clone()
+    got = trunk(z0.clone(), z_inputs, z_lm, pm, num_recycles=1)
+    assert torch.allclose(got, z, atol=1e-10)
+    assert torch.equal(z_lm, lm_before), "the LM embedding is reused by every recycle and must not change"
+    # stacks that add nothing: the recurrence has the closed form of a geometric series,
+    # z_R = a^(R+1) z_0 + (1 + a + ... + a^R) B LN(z_inputs + z_lm)
+    _zero_linear_weights(trunk.lm_stack)
+    _zero_linear_weights(trunk.main_stack)
+    a, b = trunk.dynamics()
+    drive = torch.nn.functional.linear(trunk.layernorm_z(z_inputs + z_lm), b)
+    R = 3
+    want = a ** (R + 1) * z0 + sum(a ** r for r in range(R + 1)) * drive
+    assert torch.allclose(trunk(z0.clone(), z_inputs, z_lm, pm, num_recycles=R), want, atol=1e-10)
+
+
+def test_stream_rounding_mode_of_the_block_oracle():
+    """``stream_dtype`` rounds the residual stream after every in-place add and nothing else."""
+    x = torch.tensor([1.0, 1.0, 1.0, -3.0])
+    O._stream_add_(x, torch.tensor([2.0 ** -9, 2.0 ** -8, 3 * 2.0 ** -8, 2.0 ** -7]), torch.bfloat16)
+    # bf16 keeps 8 significant bits: below half a step -> down, ties -> even, 3 - 2^-7 is a tie at
+    # step 2^-6 between 2.984375 (odd) and 3.0 (even)
+    assert x.tolist() == [1.0, 1.0, 1.015625, -3.0]
+    y = torch.tensor([1.0])
+    O._stream_add_(y, torch.tensor([2.0 ** -9]), None)
+    assert y.item() == 1.0 + 2.0 ** -9
+    c, n = 4, 4
+    plain = _rand_init(O.PairformerBlock(c, 2), 80, std=0.3).float()
+    same = O.PairformerBlock(c, 2, stream_dtype=torch.float32)
+    bf = O.PairformerBlock(c, 2, stream_dtype=torch.bfloat16)
+    same.load_state_dict(plain.state_dict())
+    bf.load_state_dict(plain.state_dict())
+    z = _rand((1, n, n, c), 81).float()
+    pm = torch.ones(1, n, n)
+    want = plain(z.clone(), pm)
+    assert torch.equal(same(z.clone(), pm), want)
+    z_bf = z.clone()
+    got = bf(z_bf, pm)
+    assert torch.equal(z_bf.to(torch.bfloat16).float(), z_bf), "the stream holds bf16 values after the block"
+    d = (got - want).abs().max().item()
+    assert 0 < d < 0.1, "rounding moves the result, by roundings only"
+    # a block that adds nothing returns the input rounded once
+    _zero_linear_weights(bf)
+    assert torch.equal(bf(z.clone(), pm), z.to(torch.bfloat16).float())
