@@ -227,3 +227,40 @@ def test_recurrence_window_and_static_entry_points_check_arguments_without_gpu()
     assert rc == -1
     rc = lib.kfh_transition_forward_static(None, None, None, None, None, 10, 100, 4, 1e-5, 0, None)
     assert rc == -2
+
+
+def test_header_is_plain_c_and_a_c_caller_links(tmp_path):
+    """The boundary is a C ABI: the header compiles as strict C99 and a C program that includes it
+    links against the library and gets the documented status codes (no GPU needed for these calls)."""
+    import shutil
+    import subprocess
+
+    if shutil.which("gcc") is None:
+        pytest.skip("gcc not found")
+    lib_dir = ROOT / "kfold_amd"
+    if not (lib_dir / "libkfold_hip.so").exists():
+        pytest.fail("kfold_amd/libkfold_hip.so is not built")
+    src = tmp_path / "caller.c"
+    src.write_text(r'''
+#include "kfold_hip.h"
+#include <stdio.h>
+#include <string.h>
+int main(void) {
+    if (kfh_version() < 1) return 1;
+    if (kfh_trimul_packed_bytes(128) == 0 || kfh_trimul_packed_bytes(64) != 0) return 2;
+    if (kfh_transition_static_scratch_bytes() != (size_t)8 << 20) return 3;
+    int rc = kfh_trimul_forward(0, 0, 0, 0, 0, 0, 0, 1, 8, 64, KFH_OUTGOING, 1e-5f, KFH_BF16, 0);
+    if (rc != KFH_EUNSUPPORTED || !strstr(kfh_last_error(), "C=64")) return 4;
+    rc = kfh_trimul_forward(0, 0, 0, 0, 0, 0, 0, 1, 8, 128, KFH_OUTGOING, 1e-5f, KFH_BF16, 0);
+    if (rc != KFH_EINVAL) return 5;
+    printf("ok\n");
+    return 0;
+}
+''')
+    exe = tmp_path / "caller"
+    cmd = ["gcc", "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", f"-I{ROOT / 'include'}", str(src),
+           "-o", str(exe), f"-L{lib_dir}", "-l:libkfold_hip.so", f"-Wl,-rpath,{lib_dir}"]
+    done = subprocess.run(cmd, capture_output=True, text=True)
+    assert done.returncode == 0, done.stderr
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0 and run.stdout.strip() == "ok", (run.returncode, run.stdout, run.stderr)
