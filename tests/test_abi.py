@@ -1,6 +1,5 @@
 """The C-ABI library loads without a GPU and exports every symbol include/kfold_hip.h declares."""
 
-import ctypes
 import re
 from pathlib import Path
 

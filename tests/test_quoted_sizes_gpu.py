@@ -19,7 +19,7 @@ import pytest
 import torch
 
 from kfold_amd import synthetic
-from tests.test_block_gpu import check_stagewise, pair_stages
+from tests.test_block_gpu import check_stagewise
 from tests.util import assert_close, assert_stream_close
 
 pytestmark = pytest.mark.gpu

@@ -84,7 +84,6 @@ def test_pair_bias_projection_and_trunk_apb(n):
         assert_close(got, want, "apb module, dense bias", auto_scale=True)
         # fused: bias tiles straight from z
         from kfold_amd import ops
-        from kfold_amd.layers.attention_pair_bias import _parameters
         tiles_dense = ops.bias_tiles_from_dense(bias.to(DEV).contiguous())
         blob = ops.pair_bias_pack(ref.layernorm_z.weight, ref.layernorm_z.bias,
                                   ref.linear_pair_bias.weight, device=torch.device(DEV))
