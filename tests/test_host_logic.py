@@ -276,3 +276,62 @@ def test_other_widths_take_the_generic_entry_points(rec):
     assert tm[7:11] == (2, 8, 256, 1)
     ta = rec.of("kfh_triattn_forward")[0]
     assert ta[7:12] == (2, 8, 64, 4, 1)
+
+
+def test_pair_bias_attention_sharing_flags(rec):
+    """Leading dimensions are flattened to samples; a bias, mask or conditioning tensor whose
+    leading dimensions are all 1 is passed once and flagged as shared (reference shapes of the
+    diffusion call site: a [B, S, L, C], s [B, S, L, Cs], bias [B, 1, H, L, L], mask [B, 1, L];
+    layers/folding/attention_pair_bias.py:114-158)."""
+    from kfold_amd import layers
+
+    S, L, C, H, Cs = 5, 40, 768, 16, 384
+    att = layers.SelfAttentionPairBias(C, H, Cs, "diffusion_global").eval()
+    a = torch.zeros(1, S, L, C, dtype=torch.bfloat16)
+    s = torch.zeros(1, S, L, Cs, dtype=torch.bfloat16)
+    bias = torch.zeros(1, 1, H, L, L, dtype=torch.bfloat16)
+    mask = torch.ones(1, 1, L, dtype=torch.bool)
+    with torch.no_grad():
+        out = att(a, s, bias, mask)
+        assert out.shape == a.shape
+        # per-sample bias and mask
+        att(a, s, bias.expand(1, S, H, L, L), mask.expand(1, S, L))
+        with pytest.raises(AssertionError):
+            att(a, None, bias, mask)
+    shared, per_sample = rec.of("kfh_apb_forward")
+    # a, s_cond, tiles, mask, blob, residual, out, ws, ws_bytes, S, L, C, H, Cs, norm, bias/mask/s per sample
+    assert shared[9:15] == (S, L, C, H, Cs, 1) and shared[15:18] == (0, 0, 1) and shared[1]
+    assert per_sample[15:18] == (1, 1, 1)
+    dense = rec.of("kfh_bias_tiles_from_dense")
+    assert dense[0][3:6] == (1, H, L) and dense[1][3:6] == (S, H, L)
+    # functional entry of the trunk call site: input already normalised, no conditioning, no norm
+    plain = layers.SelfAttentionPairBias(384, 16, None, "confidence").eval()
+    x = torch.zeros(2, L, 384, dtype=torch.bfloat16)
+    with torch.no_grad():
+        layers.hip_attention_pair_bias(plain, x, x, torch.zeros(2, 16, L, L, dtype=torch.bfloat16),
+                                       torch.ones(2, L, dtype=torch.bool))
+        with pytest.raises(NotImplementedError):
+            layers.hip_attention_pair_bias(plain, x, x.clone(), torch.zeros(2, 16, L, L), torch.ones(2, L))
+    fn = rec.of("kfh_apb_forward")[-1]
+    assert fn[9:15] == (2, L, 384, 16, 0, 0) and fn[15:18] == (1, 1, 0) and fn[1] is None
+
+
+def test_transition_rows_and_mask_plumbing(rec):
+    from kfold_amd import layers
+
+    tr = layers.Transition(128, 2).eval()
+    tr.layernorm.eps = 2e-6
+    x = torch.zeros(2, 6, 6, 128, dtype=torch.float32)
+    with torch.no_grad():
+        y = tr(x)
+    assert y.shape == x.shape and y.dtype == x.dtype
+    c = rec.of("kfh_transition_forward")[0]
+    assert c[0] == x.data_ptr() and c[2] is None and c[3] is None and c[4] == y.data_ptr() != x.data_ptr()
+    assert (c[7], c[8], c[9], c[11]) == (72, 128, 2, 1) and c[10] == pytest.approx(2e-6)
+    assert c[5] is None and c[6] == 0, "the fused C=128 kernel needs no workspace"
+    wide = layers.Transition(384, 4).eval()
+    s = torch.zeros(3, 10, 384, dtype=torch.bfloat16)
+    with torch.no_grad():
+        wide(s)
+    c = rec.of("kfh_transition_forward")[1]
+    assert (c[7], c[8], c[9], c[11]) == (30, 384, 4, 0) and c[5] and c[6] > 0
