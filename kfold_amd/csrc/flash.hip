@@ -174,7 +174,7 @@ constexpr int kStripWaves = 12;          // 768 threads, 3 wavefronts per SIMD, 
 constexpr int kStripMaxBlocks = 38;      // 38 * 4 KiB strip + scratch <= 160 KiB LDS
 
 __global__ __launch_bounds__(kStripWaves * 64, 3) void flash_strip_kernel(FlashArgs p) {
-    extern __shared__ __attribute__((aligned(16))) char lds[];
+    HIP_DYNAMIC_SHARED(__attribute__((aligned(16))) char, lds)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
     const int nb = p.nb, H = p.H;

@@ -1,0 +1,68 @@
+"""The GPU parity tests, run on the CPU through the host execution model of the kernels.
+
+Every ``test_*`` function of the ``*_gpu`` test modules gets a twin here that runs the same body
+with ``DEV = "cpu"`` while ``tests.hostsim.host_backend()`` routes the product's Python layer to
+``libkfold_hostsim.so`` — the kernel sources themselves, compiled for the host, lanes as fibers,
+MFMA / shuffles / barriers as rendezvous, workspaces between guard pages and pre-filled with NaN.
+So module → functional layer → C ABI → kernel code is compared with the oracle exactly as on the
+GPU, minus what only hardware can show (timing, memory-ordering between lanes of a wavefront).
+
+Cases that need a device (streams, CPU-tensor rejection) or more CPU time than a unit suite
+should take are listed in ``SKIP`` with the reason; the big ones carry the ``slow`` marker's
+twin in ``tests/hostsim/run_quoted_sizes.py`` instead.
+"""
+
+from __future__ import annotations
+
+import contextlib
+import functools
+import importlib
+
+import pytest
+import torch
+
+from tests import hostsim
+
+GPU_MODULES = [
+    "tests.test_trimul_gpu",
+    "tests.test_triattn_gpu",
+    "tests.test_single_track_gpu",
+    "tests.test_block_gpu",
+    "tests.test_shipping_dims_gpu",
+    "tests.test_parcae_gpu",
+    "tests.test_zz_no_alloc",
+]
+
+# test name (or "name[param id]") -> reason it has no CPU twin
+SKIP: dict[str, str] = {
+    "test_cpu_tensors_are_rejected": "the twin runs on CPU tensors by design",
+    "test_triattn_long_sequence_sampled_rows": "N = 1248 takes two minutes of CPU time "
+                                               "(tests/hostsim/run_quoted_sizes.py runs it)",
+}
+
+
+@contextlib.contextmanager
+def _on_host(mod):
+    saved = mod.DEV
+    mod.DEV = hostsim.HostDevice("cpu")
+    try:
+        with hostsim.host_backend():
+            yield
+    finally:
+        mod.DEV = saved
+
+
+def _twin(mod, fn):
+    @functools.wraps(fn)
+    def run(*args, **kwargs):
+        with _on_host(mod):
+            return fn(*args, **kwargs)
+    return run
+
+
+for _name in GPU_MODULES:
+    _mod = importlib.import_module(_name)
+    _short = _name.rsplit(".", 1)[1].replace("test_", "").replace("_gpu", "")
+    for _attr, _fn in list(vars(_mod).items()):
+        if _attr.startswith("test_") and callable(_fn) and _attr not in SKIP:
+            globals()[f"test_host_{_short}__{_attr[5:]}"] = _twin(_mod, _fn)

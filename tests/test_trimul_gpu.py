@@ -109,6 +109,11 @@ def test_trimul_weight_cache_invalidation_and_errors():
     with pytest.raises(RuntimeError):                # inference-only, like the triton backend
         with torch.enable_grad():
             hip(zd, md)
+
+
+def test_cpu_tensors_are_rejected():
+    _, hip = _modules("incoming", seed=9)
+    z, _, pm = synthetic.pair_inputs(32, 128, 0, seed=4)
     with torch.no_grad(), pytest.raises(RuntimeError):
         hip(z.to(torch.bfloat16), pm)                # CPU tensor
 
@@ -131,7 +136,8 @@ def test_caller_workspace_shared_by_consecutive_ops():
     with torch.no_grad():
         want_tm, want_ta = tm(zd, md), ta(zd, md)            # packs the weights, allocates per call
         need = max(ops.workspace_bytes("trimul", N=n, C=128), ops.workspace_bytes("triattn", N=n, C=128, heads=4))
-        ws = torch.full((need,), 0xA5, dtype=torch.uint8, device=DEV)
+        raw = torch.full((need + 256,), 0xA5, dtype=torch.uint8, device=DEV)
+        ws = raw[(-raw.data_ptr()) % 256:][:need]        # the library asks for 256-byte alignment
         for _ in range(2):
             got_tm = ops.trimul_forward(zd, md, tm._hip_multiplication_cache, "incoming", workspace=ws)
             got_ta = ops.triattn_forward(zd, md, ta._hip_attention_cache, 4, True, workspace=ws)
