@@ -5,8 +5,9 @@
 the C ABI of ``include/kfold_hip.h`` with host pointers.  ``host_backend()`` points the product's
 Python layer at that library for the duration of a test, so the modules, the functional layer, the
 C ABI and the kernel code itself run on CPU tensors and can be compared with the oracle without a
-GPU.  Workspaces handed out inside the context lie between inaccessible pages and are filled with
-NaN patterns; ``guarded()`` gives test inputs and outputs the same protection.
+GPU.  Everything the functional layer allocates inside the context (workspaces, outputs, packed
+weights, bias tiles) lies between inaccessible pages and starts out as NaN patterns; the arena the
+context yields gives test inputs the same protection.
 """
 
 from __future__ import annotations
@@ -47,6 +48,10 @@ def load() -> ctypes.CDLL:
         h.hostsim_set_skip_math.argtypes = [c_int]
         h.hostsim_launch_count.restype = c_longlong
         h.hostsim_launch_count.argtypes = []
+        h.hostsim_set_fill.restype = None
+        h.hostsim_set_fill.argtypes = [c_int]
+        h.hostsim_report.restype = None
+        h.hostsim_report.argtypes = []
         h.hostsim_threads.restype = c_int
         h.hostsim_threads.argtypes = []
         _sim = h
@@ -82,6 +87,30 @@ class _Arena:
         for p in self.ptrs:
             L.hostsim_free(p)
         self.ptrs.clear()
+
+
+class _GuardedTorch:
+    """Stands where ``torch`` stands in ``kfold_amd.ops`` while the host backend is active: the
+    buffers that module allocates (outputs, packed weights, bias tiles) come from the arena —
+    between inaccessible pages, pre-filled with 0xFF — everything else is torch's."""
+
+    def __init__(self, arena: "_Arena"):
+        self._arena = arena
+
+    def __getattr__(self, name):
+        return getattr(torch, name)
+
+    def empty(self, *size, dtype=torch.float32, device=None):
+        shape = tuple(size[0]) if len(size) == 1 and isinstance(size[0], (tuple, list, torch.Size)) else size
+        n = 1
+        for d in shape:
+            n *= int(d)
+        esz = torch.empty((), dtype=dtype).element_size()
+        raw = self._arena.bytes(n * esz, 16)
+        return raw.view(dtype).view(shape) if n else torch.empty(shape, dtype=dtype)
+
+    def empty_like(self, t):
+        return self.empty(tuple(t.shape), dtype=t.dtype)
 
 
 class HostDevice(str):
@@ -122,7 +151,7 @@ def host_backend(block_stride: int = 1, block_edge: int = 0, skip_math: bool = F
         "lib": _lib._lib, "require": ops._require_cuda, "stream": ops._stream,
         "workspace": ops._workspace, "device": torch.cuda.device,
         "synchronize": torch.cuda.synchronize, "current_stream": torch.cuda.current_stream,
-        "to": torch.Tensor.to,
+        "to": torch.Tensor.to, "torch": ops.torch,
     }
     checks = []
     for name, mod in list(sys.modules.items()):
@@ -142,6 +171,7 @@ def host_backend(block_stride: int = 1, block_edge: int = 0, skip_math: bool = F
     ops._require_cuda = _cpu_device
     ops._stream = lambda dev: None
     ops._workspace = workspace
+    ops.torch = _GuardedTorch(arena)
     torch.cuda.device = lambda dev: contextlib.nullcontext()
     torch.cuda.synchronize = lambda *a, **k: None
     torch.cuda.current_stream = lambda *a, **k: _NullStream()
@@ -150,15 +180,18 @@ def host_backend(block_stride: int = 1, block_edge: int = 0, skip_math: bool = F
         mod.check_inference = check_inference
     L.hostsim_set_block_filter(block_stride, block_edge)
     L.hostsim_set_skip_math(1 if skip_math else 0)
+    L.hostsim_set_fill(0 if skip_math else 1)      # a walk over addresses needs no NaN pattern
     try:
         yield arena
     finally:
         L.hostsim_set_block_filter(1, 0)
         L.hostsim_set_skip_math(0)
+        L.hostsim_set_fill(1)
         _lib._lib = saved["lib"]
         ops._require_cuda = saved["require"]
         ops._stream = saved["stream"]
         ops._workspace = saved["workspace"]
+        ops.torch = saved["torch"]
         torch.cuda.device = saved["device"]
         torch.cuda.synchronize = saved["synchronize"]
         torch.cuda.current_stream = saved["current_stream"]

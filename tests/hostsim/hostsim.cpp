@@ -11,6 +11,7 @@
 #include "hip/hip_runtime.h"
 
 #include <signal.h>
+#include <time.h>
 #include <sys/mman.h>
 #include <unistd.h>
 
@@ -93,6 +94,7 @@ Lane* cur() { return t_cur; }
 char* dynamic_lds() { return t_worker->lds; }
 
 static std::atomic<int> g_skip_math{0};
+static std::atomic<int> g_fill{1};
 
 [[noreturn]] static void die(const char* what) {
     Lane* c = t_cur;
@@ -311,6 +313,13 @@ static void ensure_pool() {
 
 static std::mutex& g_launch_mu = *new std::mutex;
 static std::atomic<long long> g_launches{0};
+struct KernelStat { const char* name; long long launches, blocks; double seconds; };
+static std::vector<KernelStat>& g_stats = *new std::vector<KernelStat>;
+static double now_s() {
+    timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return ts.tv_sec + 1e-9 * ts.tv_nsec;
+}
 
 void launch(const char* name, dim3 grid, dim3 block, size_t dyn_lds, const std::function<void()>& body) {
     std::lock_guard<std::mutex> launch_lock(g_launch_mu);
@@ -325,6 +334,7 @@ void launch(const char* name, dim3 grid, dim3 block, size_t dyn_lds, const std::
     j.total = (long long)grid.x * grid.y * grid.z;
     if (j.total <= 0) return;
     j.pending = g_threads;
+    const double t0 = now_s();
     {
         std::lock_guard<std::mutex> lk(g_mu);
         g_job = &j;
@@ -336,6 +346,13 @@ void launch(const char* name, dim3 grid, dim3 block, size_t dyn_lds, const std::
         g_done_cv.wait(lk, [&] { return j.pending.load() == 0; });
         g_job = nullptr;
     }
+    const double dt = now_s() - t0;
+    for (KernelStat& k : g_stats)
+        if (k.name == name || strcmp(k.name, name) == 0) {
+            k.launches++; k.blocks += j.total; k.seconds += dt;
+            return;
+        }
+    g_stats.push_back({name, 1, j.total, dt});
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -409,7 +426,8 @@ __attribute__((constructor)) static void install_handler() {
 extern "C" {
 
 // `bytes` of memory whose last byte (rounded up to `align`) is followed by an inaccessible page
-// and whose first byte is preceded by one (at a distance below a page); filled with 0xFF.
+// and whose first byte is preceded by one (at a distance below a page); filled with 0xFF unless
+// hostsim_set_fill(0) was called.
 void* hostsim_alloc(size_t bytes, size_t align) {
     using namespace hostsim;
     const size_t page = (size_t)sysconf(_SC_PAGESIZE);
@@ -422,7 +440,7 @@ void* hostsim_alloc(size_t bytes, size_t align) {
     mprotect(base, page, PROT_NONE);
     mprotect(base + page + body, page, PROT_NONE);
     char* user = base + page + (body - padded);
-    memset(base + page, 0xFF, body);
+    if (hostsim::g_fill.load()) memset(base + page, 0xFF, body);
     std::lock_guard<std::mutex> lk(g_alloc_mu);
     g_allocs.push_back({base, body + 2 * page, user, bytes});
     return user;
@@ -446,7 +464,15 @@ void hostsim_set_block_filter(long long stride, long long edge) {
     hostsim::g_filter_edge = edge;
 }
 
+// 1 (default): new buffers are filled with 0xFF; 0: left as the zero pages the kernel maps
+void hostsim_set_fill(int on) { hostsim::g_fill.store(on); }
 void hostsim_set_skip_math(int on) { hostsim::g_skip_math.store(on); }
+// per-kernel launch counts and host seconds since the last call, to stderr
+void hostsim_report(void) {
+    for (const hostsim::KernelStat& k : hostsim::g_stats)
+        fprintf(stderr, "[hostsim] %-60s launches %5lld  blocks %9lld  %8.3f s\n", k.name, k.launches, k.blocks, k.seconds);
+    hostsim::g_stats.clear();
+}
 long long hostsim_launch_count(void) { return hostsim::g_launches.load(); }
 int hostsim_threads(void) { hostsim::ensure_pool(); return hostsim::g_threads; }
 
