@@ -184,6 +184,8 @@ class MultiHeadAttention(nn.Module):
         self.linear_g = LinearNoBias(c_q, c_hidden * no_heads) if gating else None
 
     def forward(self, q_x, kv_x, tri_bias, mask):
+        if getattr(self, "operand_dtype", None) is not None:
+            return self._forward_rounded_operands(q_x, kv_x, tri_bias, mask)
         h = self.no_heads
         # :246-267 — project, split heads, move heads in front of the sequence axis
         q = self.linear_q(q_x).unflatten(-1, (h, -1)).transpose(-2, -3)
@@ -200,6 +202,43 @@ class MultiHeadAttention(nn.Module):
             g = torch.sigmoid(self.linear_g(q_x)).unflatten(-1, (h, -1))
             o = o * g
         return self.linear_o(o.flatten(-2))
+
+
+    # -- what a reduced-precision matrix unit sees ------------------------------------------
+    # Same formulas, with every operand of a matrix product rounded to ``operand_dtype`` first
+    # (inputs, weights, q, k, v, the pair bias, the probabilities, the gated output), products
+    # and sums in fp32, softmax statistics in fp32 on unrounded exponentials.  Scalings are
+    # folded where a fused kernel folds them: 1/sqrt(d) and log2(e) into the query weights and
+    # log2(e) into the bias (``tri_bias`` arrives unscaled), so the softmax runs on exp2.  Used to
+    # separate operand rounding from defects when logits are large: a kernel that computes in
+    # this precision should match THIS to normal tolerances whatever the logit magnitude.
+    def _forward_rounded_operands(self, q_x, kv_x, tri_bias, mask):
+        dt = self.operand_dtype
+
+        def rnd(t):
+            return t.to(dt).to(torch.float32)
+
+        h = self.no_heads
+        log2e = 1.4426950408889634
+        xq, xk = rnd(q_x), rnd(kv_x)
+        wq = rnd(self.linear_q.weight * (log2e / math.sqrt(self.c_hidden)))
+        q = rnd(F.linear(xq, wq)).unflatten(-1, (h, -1)).transpose(-2, -3)
+        k = rnd(F.linear(xk, rnd(self.linear_k.weight))).unflatten(-1, (h, -1)).transpose(-2, -3)
+        v = rnd(F.linear(xk, rnd(self.linear_v.weight))).unflatten(-1, (h, -1)).transpose(-2, -3)
+        logits = torch.matmul(q, k.transpose(-1, -2)) + rnd(tri_bias * log2e)
+        valid = mask.bool().expand_as(logits)
+        # a row without any valid key attends uniformly (what the finite -inf of the reference
+        # gives while |logits| < 32, triangle_attention.py:328)
+        none_valid = ~valid.any(dim=-1, keepdim=True)
+        logits = torch.where(none_valid, torch.zeros_like(logits),
+                             logits.masked_fill(~valid, float("-inf")))
+        e = torch.exp2(logits - logits.amax(dim=-1, keepdim=True))
+        o = torch.matmul(rnd(e), v) / e.sum(dim=-1, keepdim=True)
+        o = o.transpose(-2, -3)
+        if self.linear_g is not None:
+            g = torch.sigmoid(F.linear(xq, rnd(self.linear_g.weight))).unflatten(-1, (h, -1))
+            o = o * g
+        return F.linear(rnd(o.flatten(-2)), rnd(self.linear_o.weight))
 
 
 class TriangleAttention(nn.Module):
@@ -233,7 +272,13 @@ class TriangleAttention(nn.Module):
             mask = mask.transpose(-1, -2)
         x = self.layer_norm(x)                               # :411
         # :416-422 — bias [*, I, J, H] -> [*, 1, H, I, J]; here I plays "query", J "key"
-        bias = self.linear(x).movedim(-1, -3).unsqueeze(-4)
+        od = getattr(self.mha, "operand_dtype", None)
+        if od is not None:      # rounded-operand mode (see MultiHeadAttention): the bias product too
+            xr = x.to(od).to(torch.float32)
+            bias = (F.linear(xr, (self.linear.weight * 1.4426950408889634).to(od).to(torch.float32))
+                    / 1.4426950408889634).movedim(-1, -3).unsqueeze(-4)
+        else:
+            bias = self.linear(x).movedim(-1, -3).unsqueeze(-4)
         mask5 = mask[..., :, None, None, :]                  # :414  [*, I, 1, 1, J]
         n_rows = x.shape[-3]
         step = self.row_chunk or n_rows

@@ -395,3 +395,48 @@ def test_stream_rounding_mode_of_the_block_oracle():
     # a block that adds nothing returns the input rounded once
     _zero_linear_weights(bf)
     assert torch.equal(bf(z.clone(), pm), z.to(torch.bfloat16).float())
+
+
+def test_rounded_operand_mode_of_triangle_attention():
+    """The rounded-operand mode restates the attention with its scalings folded into weights and
+    an exp2 softmax.  With a rounding that changes nothing (fp32 operands) it has to reproduce
+    the pinned forward — a wrong fold (log2 e, 1/sqrt d), a transposed bias or a mask slip would
+    show — for partially masked rows and both node types; with bf16 operands it has to stay
+    close at small logits (where bf16 operands cost ~1e-3) and a fully masked row must come out
+    as uniform attention."""
+    for cls in (O.TriangleAttentionStartingNode, O.TriangleAttentionEndingNode):
+        m = cls(16, 2, row_chunk=3).eval()
+        g = torch.Generator().manual_seed(31)
+        with torch.no_grad():
+            for name, p in m.named_parameters():
+                if p.dim() >= 2:
+                    p.copy_(0.5 * torch.randn(p.shape, generator=g))
+                else:
+                    p.copy_(1 + 0.2 * torch.randn(p.shape, generator=g))
+        x = torch.randn(1, 7, 7, 16, generator=g)
+        mask = torch.rand(1, 7, 7, generator=g) > 0.3
+        mask[0, :, 0] = True
+        mask[0, 0, :] = True                 # every row / column keeps a valid key
+        with torch.no_grad():
+            want = m(x, mask.float())
+            m.mha.operand_dtype = torch.float32
+            same = m(x, mask.float())
+            m.mha.operand_dtype = torch.bfloat16
+            rounded = m(x, mask.float())
+            m.mha.operand_dtype = None
+        assert torch.allclose(same, want, atol=2e-5, rtol=1e-5), (same - want).abs().max()
+        err = (rounded - want).abs().max().item()
+        assert 1e-5 < err < 0.15, err         # it does round, and only rounds
+    # fully masked row -> uniform attention over all keys
+    m = O.TriangleAttentionStartingNode(16, 2).eval()
+    _ = [torch.nn.init.normal_(p, std=0.3) for p in m.parameters() if p.dim() >= 2]
+    x = torch.randn(1, 5, 5, 16, generator=torch.Generator().manual_seed(3))
+    mask = torch.ones(1, 5, 5)
+    mask[0, 2, :] = 0
+    with torch.no_grad():
+        m.mha.operand_dtype = torch.float32
+        got = m(x, mask)[0, 2]
+        xn = m.layer_norm(x)[0, 2]
+        v_mean = m.mha.linear_v(xn).mean(dim=0, keepdim=True)
+        uniform = m.mha.linear_o(torch.sigmoid(m.mha.linear_g(xn)) * v_mean)
+    assert torch.allclose(got, uniform, atol=1e-5)

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from kfold_amd import synthetic
-from tests.util import assert_close
+from tests.util import assert_close, errors
 
 pytestmark = pytest.mark.gpu
 
@@ -140,20 +140,28 @@ def test_triattn_logits_far_from_zero(shift):
 
 
 def test_triattn_fully_masked_rows_with_large_varying_logits():
-    """Rows whose keys are all masked (padded query rows; the block's final mask zeroes them).
-    The reference adds a finite -1e9 to every masked logit in fp32 (triangle_attention.py:328):
+    """Large logits (|q.k| beyond 100) and rows whose keys are all masked.
+
+    Rows with a valid key: at logits this size the rounding of the MFMA operands to bf16 (2^-9
+    relative on q and k, i.e. a few tenths in an exponent of 100) moves the result away from an
+    all-fp32 evaluation by far more than the benchmark tolerance.  That this is operand rounding
+    and nothing else is shown by the oracle's rounded-operand mode (same formulas, every matrix
+    operand rounded to bf16, fp32 sums): it is as far from the fp32 oracle as the kernel is, and
+    the kernel matches IT at the unscaled limits.
+
+    Rows whose keys are all masked (padded query rows; the block's final mask zeroes them):
+    the reference adds a finite -1e9 to every masked logit in fp32 (triangle_attention.py:328):
     the spacing of fp32 at 1e9 is 64, so logits below 32 in magnitude vanish in that sum and the
     row attends uniformly, while larger ones leave a residue that is a multiple of 64 (weights
     then differ by factors of e^64 and flip with the last bit of q.k).  The kernel attends
     uniformly over the N keys in every fully masked row, whatever the logits: identical to the
-    reference while |q.k|, |bias| < 32, a stated deviation beyond.  Rows with a valid key follow
-    the reference at any logit size."""
+    reference while |q.k|, |bias| < 32, a stated deviation beyond."""
     print("case triattn fully masked rows, large varying logits", flush=True)
     ref, hip = _modules(True, seed=21, std=0.02)
     g = torch.Generator().manual_seed(22)
     with torch.no_grad():
         for w in (ref.mha.linear_q.weight, ref.mha.linear_k.weight):
-            w.copy_(0.25 * torch.randn(w.shape, generator=g))       # |q.k| reaches ~40
+            w.copy_(0.5 * torch.randn(w.shape, generator=g))        # |q.k| reaches ~150
         ref.linear.weight.copy_(0.5 * torch.randn(ref.linear.weight.shape, generator=g))
         for w in (ref.mha.linear_v.weight, ref.mha.linear_o.weight, ref.mha.linear_g.weight):
             w.copy_(0.1 * torch.randn(w.shape, generator=g))
@@ -167,14 +175,22 @@ def test_triattn_fully_masked_rows_with_large_varying_logits():
     with torch.no_grad():
         got = hip(xb.to(DEV), mask.to(DEV)).float().cpu()
         want = ref(xb.float(), mask.float())
+        ref.mha.operand_dtype = torch.bfloat16
+        want_rounded = ref(xb.float(), mask.float())
+        ref.mha.operand_dtype = None
         xn = ref.layer_norm(xb.float())
         q = ref.mha.linear_q(xn[0, dead]).unflatten(-1, (4, 32)) / 32 ** 0.5
         k = ref.mha.linear_k(xn[0, dead]).unflatten(-1, (4, 32))
         assert torch.einsum("rqhd,rkhd->rhqk", q, k).abs().max() > 32     # residues do occur
         live = [i for i in range(n) if i not in dead]
-        # (bf16 operands at logits of this size: only the relative gate is meaningful)
-        assert_close(got[0, live], want[0, live], "rows with a valid key, large logits",
-                     max_abs=float("inf"), mean_abs=float("inf"), rel_fro=4e-2)
+        e_f32 = errors(got[0, live], want[0, live])
+        e_model = errors(want_rounded[0, live], want[0, live])
+        print(f"  kernel vs fp32 oracle {e_f32}\n  rounded-operand oracle vs fp32 oracle {e_model}", flush=True)
+        # operand rounding alone costs what the kernel is off by ...
+        assert e_model["max_abs"] > 5 * 2e-2 and e_f32["max_abs"] < 1.5 * e_model["max_abs"]
+        # ... and against the same arithmetic the kernel meets the unscaled limits
+        print(assert_close(got[0, live], want_rounded[0, live], "rows with a valid key, large logits, "
+                           "against the rounded-operand oracle"), flush=True)
         # fully masked rows: gate * mean of v over all N keys, projected
         v_mean = ref.mha.linear_v(xn[0, dead]).mean(dim=1, keepdim=True)           # [rows, 1, 128]
         gate = torch.sigmoid(ref.mha.linear_g(xn[0, dead]))                         # [rows, N, 128]
