@@ -14,6 +14,7 @@ import sys
 import time
 
 import tests.test_quoted_sizes_gpu as Q
+import tests.test_shipping_dims_gpu as SD
 import tests.test_triattn_gpu as TA
 from tests import hostsim
 from tests.test_hostsim_parity import _on_host
@@ -26,6 +27,8 @@ CASES = [
     (Q, "test_apb_diffusion_variant_n768", [(False,), (True,)]),
     (Q, "test_block_n768_metric_shape", [()]),
     (TA, "test_triattn_long_sequence_sampled_rows", [()]),
+    (SD, "test_triattn_c64_templates_n384", [(True,), (False,)]),
+    (SD, "test_trimul_c256_tiled_sizes", [(384, "outgoing"), (384, "incoming"), (768, "outgoing"), (768, "incoming")]),
 ]
 
 

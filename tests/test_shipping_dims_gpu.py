@@ -119,3 +119,60 @@ def test_triattn_other_widths_batched(starting, c, h, n, batch):
         xin = xd.clone()
         ops.triattn_forward(xin, md, hip._hip_attention_cache, h, starting, residual=xin, out=xin)
         assert_close(xin, x.float() + want, "residual in place", rel_fro=5e-3, auto_scale=True)
+
+
+@pytest.mark.parametrize("direction", ["outgoing", "incoming"])
+@pytest.mark.parametrize("n", [384, 768])
+def test_trimul_c256_tiled_sizes(direction, n):
+    """C = 256 at sizes whose padded planes take the 256 x 256 contraction tiles (N = 130 and
+    below run on 128 x 128 tiles only) with 12 % padding; the oracle's einsum in full."""
+    from kfold_amd import primitives as P
+    from oracle import torch_path as O
+
+    print(f"case trimul C=256 {direction} n={n}", flush=True)
+    cls = "TriangleMultiplicationOutgoing" if direction == "outgoing" else "TriangleMultiplicationIncoming"
+    ref = getattr(O, cls)(256).eval()
+    synthetic.init_weights_(ref, 5)
+    hip = getattr(P, cls)(256).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    z, _, pm = synthetic.pair_inputs(n, 256, synthetic.n_pad_for(n, 0.12), seed=n + 1)
+    zb = z.bfloat16()
+    with torch.no_grad():
+        want = ref(zb.float(), pm)
+        got = hip(zb.to(DEV), pm.to(DEV))
+    print(assert_close(got, want, f"trimul C=256 {direction} n={n}"), flush=True)
+    assert (got.cpu()[~pm] == 0).all()
+
+
+@pytest.mark.parametrize("starting", [True, False])
+def test_triattn_c64_templates_n384(starting):
+    """The template stack's shape at a realistic length: c = 64, 4 heads x 16, 4 templates,
+    N = 384 (12 key blocks; the bias of each template is its own).  Oracle on sampled rows of
+    every template."""
+    from kfold_amd import primitives as P
+    from oracle import torch_path as O
+
+    print(f"case triattn c=64 templates n=384 starting={starting}", flush=True)
+    n, batch = 384, 4
+    cls = "TriangleAttentionStartingNode" if starting else "TriangleAttentionEndingNode"
+    ref = getattr(O, cls)(64, 4).eval()
+    synthetic.init_weights_(ref, 17, std=0.08)
+    hip = getattr(P, cls)(64, 4).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(batch, n, n, 64, generator=g).bfloat16()
+    masks = [synthetic.pair_mask_from_tokens(synthetic.token_mask(n, pad))[0] for pad in (0, 46, 7, 100)]
+    mask = torch.stack(masks)
+    rows = [0, 31, 32, 200, 283, 284, 337, 338, 383]
+    with torch.no_grad():
+        got = hip(x.to(DEV), mask.to(DEV)).float().cpu()
+        for b in range(batch):
+            xt = x[b:b + 1].float() if starting else x[b:b + 1].float().transpose(1, 2)
+            mt = mask[b:b + 1].float() if starting else mask[b:b + 1].float().transpose(1, 2)
+            xn = ref.layer_norm(xt)
+            bias = ref.linear(xn).movedim(-1, -3).unsqueeze(-4)
+            want = ref.mha(xn[:, rows], xn[:, rows], bias, mt[..., :, None, None, :][:, rows])[0]
+            gb = (got[b] if starting else got[b].transpose(0, 1))[rows]
+            print(assert_close(gb, want, f"triattn c=64 template {b}", auto_scale=True), flush=True)
