@@ -13,8 +13,14 @@
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); every call
  *     only enqueues work on it and never synchronises;
  *   - `io_dtype` / `w_dtype` select the element type of activations / source weights:
- *     KFH_BF16 (0) or KFH_F32 (1).  Arithmetic is always bf16 MFMA with fp32
- *     accumulation and fp32 LayerNorm / softmax statistics;
+ *     KFH_BF16 (0) or KFH_F32 (1).  Arithmetic is bf16 MFMA with fp32 accumulation and fp32
+ *     LayerNorm / softmax statistics (what the reference computes under its bf16 autocast,
+ *     inference/runner.py:565-571); the pair-bias attention entry points also take
+ *     `arith` = KFH_ARITH_F32 for the fp32 arithmetic the reference's diffusion stack runs in
+ *     (model/model.py:419, fp32_dot_precision="ieee" in
+ *     kernels/triton/attention_pair_bias/dispatch.py:439,453): every product is then carried
+ *     to fp32 accuracy on the bf16 matrix cores by splitting each fp32 operand into three
+ *     bf16 parts (six part products per k-step);
  *   - masks are one byte per element, non-zero = valid;
  *   - inputs are only read; `out` must not overlap an input unless the entry point says
  *     so (the `residual` arguments may alias `out`);
@@ -35,6 +41,11 @@ extern "C" {
 
 #define KFH_BF16 0
 #define KFH_F32 1
+
+/* arithmetic of the pair-bias attention entry points; blobs, bias tiles and workspaces of one
+ * arithmetic cannot be used with the other */
+#define KFH_ARITH_BF16 0 /* bf16 operands, fp32 accumulation (bf16 autocast of the reference)   */
+#define KFH_ARITH_F32 1  /* fp32-accurate products ("ieee"), for fp32 activations and weights   */
 
 #define KFH_OK 0
 #define KFH_EINVAL (-1)      /* bad argument (shape, dtype, null pointer, small workspace) */
@@ -160,21 +171,23 @@ int kfh_transition_forward_static(const void* x, const void* blob, const void* r
                                   float eps, int io_dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------
- * Pair bias of the token-track attention, as bf16 "bias tiles": the layout the attention
- * kernel reads, [batch][head][query block of 32][key block of 32][2 KiB tile], values
- * pre-multiplied by log2(e); inside a tile the 1024 values are in the register order of the
- * kernel's transposed score accumulator (an opaque layout: produce tiles only with the two
+ * Pair bias of the token-track attention, as "bias tiles": the layout the attention
+ * kernel reads, [batch][head][query block of 32][key block of 32][tile], values
+ * pre-multiplied by log2(e); a tile is 2 KiB of bf16 (KFH_ARITH_BF16) or 4 KiB of fp32
+ * (KFH_ARITH_F32); inside a tile the 1024 values are in the register order of the
+ * kernel's transposed score accumulator (an opaque layout: produce tiles only with the
  * calls below).
  * ------------------------------------------------------------------------------------- */
-size_t kfh_bias_tiles_bytes(int nbatch, int H, int L);
+size_t kfh_bias_tiles_bytes(int nbatch, int H, int L, int arith);
 
 /* tiles <- dense pair bias [nbatch, H, L, L] (io_dtype), the `pair_bias` argument of
  * model/primitives/attention.py:28-37. */
 int kfh_bias_tiles_from_dense(const void* dense, int io_dtype, void* tiles, int nbatch, int H, int L,
-                              void* stream);
+                              int arith, void* stream);
 
 /* tiles <- linear_pair_bias(layernorm_z(z)) moved to [B, H, N, N]
- * (model/modules/confidence_head.py:162-163) in one pass over z [B, N, N, C]; w is [H, C]. */
+ * (model/modules/confidence_head.py:162-163) in one pass over z [B, N, N, C]; w is [H, C].
+ * bf16 tiles (KFH_ARITH_BF16): the confidence head and trunk run under autocast. */
 size_t kfh_pair_bias_packed_bytes(int C, int H);
 int kfh_pair_bias_pack(const void* ln_w, const void* ln_b, const void* w, int w_dtype, int C, int H,
                        void* blob, void* stream);
@@ -189,7 +202,7 @@ int kfh_pair_bias_project(const void* z, const void* blob, void* tiles, int B, i
  * math of the torch path at attention.py:75-94, :239-271, :122-168.
  * C = channel_a, H heads of C/H (<= 64) channels, Cs = conditioning channels (0 = none).
  * ------------------------------------------------------------------------------------- */
-size_t kfh_apb_packed_bytes(int C, int H, int Cs);
+size_t kfh_apb_packed_bytes(int C, int H, int Cs, int arith);
 
 /* q_w,k_w,v_w,g_w,o_w [C, C]; q_b [C] or NULL (`linear_q.bias`); unconditioned: ln_w, ln_b [C]
  * (`layernorm_a`); conditioned (Cs > 0): adaln_s_w [Cs] (`adaln_a.layernorm_s.weight`),
@@ -199,9 +212,9 @@ int kfh_apb_pack(const void* ln_w, const void* ln_b, const void* q_w, const void
                  const void* v_w, const void* g_w, const void* o_w, const void* adaln_s_w,
                  const void* adaln_g_w, const void* adaln_g_b, const void* adaln_bias_w,
                  const void* ada_out_w, const void* ada_out_b, int w_dtype, int C, int H, int Cs,
-                 void* blob, void* stream);
+                 int arith, void* blob, void* stream);
 
-size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs);
+size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs, int arith);
 
 /* a, out, residual: [S, L, C]; s_cond: [S or 1, L, Cs]; bias_tiles: [S or 1] batches of tiles;
  * mask: [S or 1, L] bytes (valid keys); the *_per_sample flags say which of the two.
@@ -209,12 +222,13 @@ size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs);
  * conditioning gate is applied; apply_norm != 0: LayerNorm (Cs = 0) or AdaLN + the
  * sigmoid(linear_ada_out(s)) output gate (Cs > 0) are applied as the module does.
  * out = (residual or 0) + result; `residual` may alias `out`, `out` must not alias `a`
- * unless residual == a.  Fully masked key sets give uniform attention (finite -1e9). */
+ * unless residual == a.  Fully masked key sets give uniform attention (finite -1e9).
+ * `arith` must be the one the blob, the bias tiles and the workspace size were made for. */
 int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, const uint8_t* mask,
                     const void* blob, const void* residual, void* out, void* workspace,
                     size_t workspace_bytes, int S, int L, int C, int H, int Cs, int apply_norm,
                     int bias_per_sample, int mask_per_sample, int s_per_sample, float eps,
-                    int io_dtype, void* stream);
+                    int io_dtype, int arith, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Cross attention with pair bias over local windows: the whole
@@ -222,11 +236,10 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
  * model/primitives/attention.py:75-94, :239-271) of the atom transformer: W windows, each with
  * Lq queries (32) attending to Lk keys (128) under its own bias [H, Lq, Lk] and key mask [Lk].
  * C = channel_a (a multiple of 32), H heads of C/H <= 64 channels, Cs = conditioning channels
- * (0 = none, else a multiple of 16).  Arithmetic is bf16 MFMA / fp32 accumulation like every
- * other entry point; the fp32 ("ieee") arithmetic the reference selects for its diffusion
- * stack (model/model.py:419) is not built.
+ * (0 = none, else a multiple of 16).  `arith` as for kfh_apb_*: KFH_ARITH_F32 is the fp32
+ * ("ieee") arithmetic the reference selects for its diffusion stack (model/model.py:419).
  * ------------------------------------------------------------------------------------- */
-size_t kfh_cross_apb_packed_bytes(int C, int H, int Cs);
+size_t kfh_cross_apb_packed_bytes(int C, int H, int Cs, int arith);
 
 /* unconditioned: lnq_*, lnk_* [C] (`layernorm_a_q`, `layernorm_a_k`); conditioned: adaq_* / adak_*
  * are `adaln_a_q` / `adaln_a_k` (`layernorm_s.weight` [Cs], `linear_g` [C, Cs] + bias [C],
@@ -236,18 +249,25 @@ int kfh_cross_apb_pack(const void* lnq_w, const void* lnq_b, const void* lnk_w, 
                        const void* o_w, const void* adaq_s_w, const void* adaq_g_w, const void* adaq_g_b,
                        const void* adaq_bias_w, const void* adak_s_w, const void* adak_g_w,
                        const void* adak_g_b, const void* adak_bias_w, const void* ada_out_w,
-                       const void* ada_out_b, int w_dtype, int C, int H, int Cs, void* blob, void* stream);
+                       const void* ada_out_b, int w_dtype, int C, int H, int Cs, int arith, void* blob,
+                       void* stream);
 
-size_t kfh_cross_apb_workspace_bytes(int W, int Lq, int Lk, int C, int H, int Cs);
+size_t kfh_cross_apb_workspace_bytes(int W, int Lq, int Lk, int C, int H, int Cs, int arith);
 
 /* a_q, out, residual: [W, Lq, C]; a_k: [W, Lk, C]; s_q: [W, Lq, Cs], s_k: [W, Lk, Cs] (Cs > 0);
  * pair_bias: dense [W, H, Lq, Lk] of bias_dtype; mask: [W, Lk] bytes.
+ * apply_norm != 0: the whole module (LayerNorm or AdaLN of both sides, attention, and with
+ * Cs > 0 the sigmoid(linear_ada_out(s_q)) output gate); apply_norm = 0: a_q / a_k are already
+ * normalised and s_q / s_k are ignored — the functional entry `attention_pair_bias(module, x_q,
+ * x_k, ...)` of model/primitives/attention.py:28-94 with x_q != x_k, as
+ * CrossAttentionPairBias.forward calls it (attention_pair_bias.py:250-258).
  * out = (residual or 0) + result; `residual` may alias `out`.  A window whose keys are all
  * masked attends uniformly over its Lk keys (finite -1e9). */
 int kfh_cross_apb_forward(const void* a_q, const void* a_k, const void* s_q, const void* s_k,
                           const void* pair_bias, int bias_dtype, const uint8_t* mask, const void* blob,
                           const void* residual, void* out, void* workspace, size_t workspace_bytes, int W,
-                          int Lq, int Lk, int C, int H, int Cs, float eps, int io_dtype, void* stream);
+                          int Lq, int Lk, int C, int H, int Cs, int apply_norm, float eps, int io_dtype,
+                          int arith, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Parcae recurrence step of the trunk: replaces the torch line

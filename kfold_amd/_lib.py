@@ -15,6 +15,7 @@ LIB_PATH = Path(__file__).resolve().parent / "libkfold_hip.so"
 KFH_BF16, KFH_F32 = 0, 1
 KFH_OUTGOING, KFH_INCOMING = 0, 1
 KFH_STAGE_IN, KFH_STAGE_CORE, KFH_STAGE_OUT, KFH_STAGE_ALL = 1, 2, 4, 7
+KFH_ARITH_BF16, KFH_ARITH_F32 = 0, 1
 
 # name -> (restype, argtypes); mirrors include/kfold_hip.h one to one
 _P = c_void_p
@@ -42,21 +43,21 @@ SIGNATURES: dict[str, tuple] = {
                                        c_float, c_int, _P]),
     "kfh_transition_static_scratch_bytes": (c_size_t, []),
     "kfh_transition_forward_static": (c_int, [_P, _P, _P, _P, _P, c_longlong, c_int, c_int, c_float, c_int, _P]),
-    "kfh_bias_tiles_bytes": (c_size_t, [c_int, c_int, c_int]),
-    "kfh_bias_tiles_from_dense": (c_int, [_P, c_int, _P, c_int, c_int, c_int, _P]),
+    "kfh_bias_tiles_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "kfh_bias_tiles_from_dense": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P]),
     "kfh_pair_bias_packed_bytes": (c_size_t, [c_int, c_int]),
     "kfh_pair_bias_pack": (c_int, [_P, _P, _P, c_int, c_int, c_int, _P, _P]),
     "kfh_pair_bias_project": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
-    "kfh_apb_packed_bytes": (c_size_t, [c_int, c_int, c_int]),
-    "kfh_apb_pack": (c_int, [_P] * 14 + [c_int, c_int, c_int, c_int, _P, _P]),
-    "kfh_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "kfh_apb_packed_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "kfh_apb_pack": (c_int, [_P] * 14 + [c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "kfh_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
     "kfh_apb_forward": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
-                                c_int, c_int, c_int, c_int, c_int, c_float, c_int, _P]),
-    "kfh_cross_apb_packed_bytes": (c_size_t, [c_int, c_int, c_int]),
-    "kfh_cross_apb_pack": (c_int, [_P] * 20 + [c_int, c_int, c_int, c_int, _P, _P]),
-    "kfh_cross_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+                                c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P]),
+    "kfh_cross_apb_packed_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "kfh_cross_apb_pack": (c_int, [_P] * 20 + [c_int, c_int, c_int, c_int, c_int, _P, _P]),
+    "kfh_cross_apb_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int, c_int]),
     "kfh_cross_apb_forward": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, _P, c_size_t, c_int, c_int,
-                                      c_int, c_int, c_int, c_int, c_float, c_int, _P]),
+                                      c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, _P]),
     "kfh_parcae_packed_bytes": (c_size_t, [c_int]),
     "kfh_parcae_pack": (c_int, [_P, _P, _P, _P, _P, c_int, c_int, _P, _P]),
     "kfh_parcae_step": (c_int, [_P, _P, _P, _P, _P, c_longlong, c_int, c_float, c_int, _P]),

@@ -19,13 +19,18 @@ using namespace kfh;
 namespace {
 
 // ---- blob / workspace layouts -------------------------------------------------------------
+// parts = 1: bf16 arithmetic; parts = 3 (KFH_ARITH_F32): every packed matrix and every bf16
+// intermediate is stored as its three split3 planes, one after the other
 struct ApbLayout {
-    int C, H, Dh, PB, Cs, kq, nhb, ko;
+    int C, H, Dh, PB, Cs, kq, nhb, ko, parts;
     size_t wq, wk, wv, wg, wo, w_adag, w_adab, w_adaout, f_bq, f_ln_g, f_ln_b, f_lns_g, f_adag_b,
         f_adaout_b, total;
+    size_t wh, wo_bytes, wa;          // bytes of one part of a head projection / the output projection / an AdaLN matrix
     bool ok;
-    ApbLayout(int C_, int H_, int Cs_) : C(C_), H(H_), Cs(Cs_) {
-        ok = C > 0 && H > 0 && C % H == 0 && C % 128 == 0 && C <= 2048 && (Cs == 0 || (Cs % 128 == 0 && Cs <= 2048));
+    ApbLayout(int C_, int H_, int Cs_, int arith = KFH_ARITH_BF16) : C(C_), H(H_), Cs(Cs_) {
+        parts = arith == KFH_ARITH_F32 ? 3 : 1;
+        ok = (arith == KFH_ARITH_BF16 || arith == KFH_ARITH_F32) && C > 0 && H > 0 && C % H == 0 && C % 128 == 0 &&
+             C <= 2048 && (Cs == 0 || (Cs % 128 == 0 && Cs <= 2048));
         if (!ok) { total = 0; return; }
         Dh = C / H;
         PB = (Dh + 31) / 32;
@@ -36,11 +41,12 @@ struct ApbLayout {
         ko = nhb * 2;
         size_t off = 0;
         auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
-        const size_t wh = (size_t)nhb * kq * 1024;
-        wq = take(wh); wk = take(wh); wv = take(wh); wg = take(wh);
-        wo = take((size_t)(C / 32) * ko * 1024);
-        const size_t wa = Cs ? (size_t)(C / 32) * (Cs / 16) * 1024 : 0;
-        w_adag = take(wa); w_adab = take(wa); w_adaout = take(wa);
+        wh = (size_t)nhb * kq * 1024;
+        wq = take(parts * wh); wk = take(parts * wh); wv = take(parts * wh); wg = take(parts * wh);
+        wo_bytes = (size_t)(C / 32) * ko * 1024;
+        wo = take(parts * wo_bytes);
+        wa = Cs ? (size_t)(C / 32) * (Cs / 16) * 1024 : 0;
+        w_adag = take(parts * wa); w_adab = take(parts * wa); w_adaout = take(parts * wa);
         f_bq = take(C * 4); f_ln_g = take(C * 4); f_ln_b = take(C * 4);
         f_lns_g = take(Cs * 4); f_adag_b = take(C * 4); f_adaout_b = take(C * 4);
         total = off;
@@ -49,19 +55,23 @@ struct ApbLayout {
 
 struct ApbWs {
     size_t xn, an, sn, sraw, gate_out, qf, kf, vf, gf, of, codes, total;
+    size_t rows_c, rows_cs, frag;     // bytes of one part of a [rows, C] / [rows, Cs] bf16 tensor / a fragment buffer
     int nb;
     ApbWs(const ApbLayout& l, int S, int L) {
         nb = (L + 31) / 32;
         size_t off = 0;
         auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
         const size_t rows = (size_t)S * L;
-        xn = take(rows * l.C * 2);
-        an = take(l.Cs ? rows * l.C * 2 : 0);
-        sn = take(l.Cs ? rows * l.Cs * 2 : 0);
-        sraw = take(l.Cs ? rows * l.Cs * 2 : 0);
-        gate_out = take(l.Cs ? rows * l.C * 2 : 0);
-        const size_t frag = (size_t)S * l.H * nb * l.PB * 2048;
-        qf = take(frag); kf = take(frag); vf = take(frag); gf = take(frag); of = take(frag);
+        const size_t P = l.parts;
+        rows_c = rows * l.C * 2;
+        rows_cs = rows * l.Cs * 2;
+        xn = take(P * rows_c);
+        an = take(l.Cs ? P * rows_c : 0);
+        sn = take(l.Cs ? P * rows_cs : 0);
+        sraw = take(l.Cs ? P * rows_cs : 0);
+        gate_out = take(l.Cs ? rows * l.C * (P == 3 ? 4 : 2) : 0);      // fp32 gate in fp32 arithmetic
+        frag = (size_t)S * l.H * nb * l.PB * 2048;
+        qf = take(P * frag); kf = take(P * frag); vf = take(P * frag); gf = take(P * frag); of = take(P * frag);
         codes = take((size_t)S * nb * 32);
         total = off;
     }
@@ -97,19 +107,25 @@ extern "C" {
 // ------------------------------------------------------------------------------------------
 // pair bias tiles
 // ------------------------------------------------------------------------------------------
-size_t kfh_bias_tiles_bytes(int nbatch, int H, int L) {
-    if (nbatch <= 0 || H <= 0 || L <= 0) return 0;
+size_t kfh_bias_tiles_bytes(int nbatch, int H, int L, int arith) {
+    if (nbatch <= 0 || H <= 0 || L <= 0 || (arith != KFH_ARITH_BF16 && arith != KFH_ARITH_F32)) return 0;
     const size_t nb = (L + 31) / 32;
-    return align_up((size_t)nbatch * H * nb * nb * 2048);
+    return align_up((size_t)nbatch * H * nb * nb * (arith == KFH_ARITH_F32 ? kBiasTileF32Bytes : 2048));
 }
 
 int kfh_bias_tiles_from_dense(const void* dense, int io_dtype, void* tiles, int nbatch, int H, int L,
-                              void* stream) {
+                              int arith, void* stream) {
     if (!dense || !tiles || nbatch <= 0 || H <= 0 || L <= 0)
         return fail(KFH_EINVAL, "bias_tiles_from_dense: bad argument");
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "bias_tiles_from_dense: bad io_dtype %d", io_dtype);
-    launch_bias_tiles(dense, io_dtype, static_cast<uint16_t*>(tiles), nbatch, H, L, (L + 31) / 32,
-                      static_cast<hipStream_t>(stream));
+    if (arith != KFH_ARITH_BF16 && arith != KFH_ARITH_F32)
+        return fail(KFH_EINVAL, "bias_tiles_from_dense: bad arith %d", arith);
+    if (arith == KFH_ARITH_F32)
+        launch_bias_tiles_f32(dense, io_dtype, static_cast<float*>(tiles), nbatch, H, L, (L + 31) / 32,
+                              static_cast<hipStream_t>(stream));
+    else
+        launch_bias_tiles(dense, io_dtype, static_cast<uint16_t*>(tiles), nbatch, H, L, (L + 31) / 32,
+                          static_cast<hipStream_t>(stream));
     return check_launch("bias_tiles_from_dense");
 }
 
@@ -154,15 +170,15 @@ int kfh_pair_bias_project(const void* z, const void* blob, void* tiles, int B, i
 // ------------------------------------------------------------------------------------------
 // pair-bias attention
 // ------------------------------------------------------------------------------------------
-size_t kfh_apb_packed_bytes(int C, int H, int Cs) { return ApbLayout(C, H, Cs).total; }
+size_t kfh_apb_packed_bytes(int C, int H, int Cs, int arith) { return ApbLayout(C, H, Cs, arith).total; }
 
 int kfh_apb_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* q_b, const void* k_w,
                  const void* v_w, const void* g_w, const void* o_w, const void* adaln_s_w,
                  const void* adaln_g_w, const void* adaln_g_b, const void* adaln_bias_w,
                  const void* ada_out_w, const void* ada_out_b, int w_dtype, int C, int H, int Cs,
-                 void* blob, void* stream_) {
-    const ApbLayout l(C, H, Cs);
-    if (!l.ok) return fail(KFH_EUNSUPPORTED, "apb_pack: C=%d H=%d Cs=%d not supported (C,Cs multiples of 128 up to 2048, head dim <= 64)", C, H, Cs);
+                 int arith, void* blob, void* stream_) {
+    const ApbLayout l(C, H, Cs, arith);
+    if (!l.ok) return fail(KFH_EUNSUPPORTED, "apb_pack: C=%d H=%d Cs=%d arith=%d not supported (C,Cs multiples of 128 up to 2048, head dim <= 64)", C, H, Cs, arith);
     if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "apb_pack: bad w_dtype %d", w_dtype);
     if (!q_w || !k_w || !v_w || !g_w || !o_w || !blob) return fail(KFH_EINVAL, "apb_pack: null pointer");
     if (Cs && (!adaln_g_w || !adaln_bias_w || !ada_out_w))
@@ -171,25 +187,31 @@ int kfh_apb_pack(const void* ln_w, const void* ln_b, const void* q_w, const void
     char* b = static_cast<char*>(blob);
     const float qscale = kLog2e / sqrtf((float)l.Dh);
     const size_t blk = (size_t)l.kq * 1024;
-    for (int h = 0; h < H; ++h)
-        for (int pp = 0; pp < l.PB; ++pp) {
-            const int rows = l.Dh - 32 * pp < 32 ? l.Dh - 32 * pp : 32;
-            const int row0 = h * l.Dh + 32 * pp;
-            const size_t o = (size_t)(h * l.PB + pp) * blk;
-            launch_pack_blocks(q_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, qscale, b + l.wq + o, stream);
-            launch_pack_blocks(k_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wk + o, stream);
-            launch_pack_blocks(v_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wv + o, stream);
-            launch_pack_blocks(g_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wg + o, stream);
+    for (int q = 0; q < l.parts; ++q) {
+        const int part = l.parts == 3 ? q : -1;
+        for (int h = 0; h < H; ++h)
+            for (int pp = 0; pp < l.PB; ++pp) {
+                const int rows = l.Dh - 32 * pp < 32 ? l.Dh - 32 * pp : 32;
+                const int row0 = h * l.Dh + 32 * pp;
+                const size_t o = (size_t)q * l.wh + (size_t)(h * l.PB + pp) * blk;
+                launch_pack_blocks(q_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, qscale, b + l.wq + o, stream, 0, part);
+                launch_pack_blocks(k_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wk + o, stream, 0, part);
+                launch_pack_blocks(v_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wv + o, stream, 0, part);
+                launch_pack_blocks(g_w, w_dtype, rows, C, C, row0, 1, ROW_NATURAL, K_NATURAL, 1.f, b + l.wg + o, stream, 0, part);
+            }
+        launch_pack_blocks(o_w, w_dtype, C, l.ko * 16, C, 0, C / 32, ROW_NATURAL, K_ACC_HEADPAD, 1.f,
+                           b + l.wo + (size_t)q * l.wo_bytes, stream, l.Dh | ((2 * l.PB) << 16), part);
+        if (Cs) {
+            const size_t oa = (size_t)q * l.wa;
+            launch_pack_blocks(adaln_g_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adag + oa, stream, 0, part);
+            launch_pack_blocks(adaln_bias_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adab + oa, stream, 0, part);
+            launch_pack_blocks(ada_out_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adaout + oa, stream, 0, part);
         }
-    launch_pack_blocks(o_w, w_dtype, C, l.ko * 16, C, 0, C / 32, ROW_NATURAL, K_ACC_HEADPAD, 1.f, b + l.wo,
-                       stream, l.Dh | ((2 * l.PB) << 16));
+    }
     launch_copy_f32(q_b, w_dtype, reinterpret_cast<float*>(b + l.f_bq), C, 0.f, stream);
     launch_copy_f32(ln_w, w_dtype, reinterpret_cast<float*>(b + l.f_ln_g), C, 1.f, stream);
     launch_copy_f32(ln_b, w_dtype, reinterpret_cast<float*>(b + l.f_ln_b), C, 0.f, stream);
     if (Cs) {
-        launch_pack_blocks(adaln_g_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adag, stream);
-        launch_pack_blocks(adaln_bias_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adab, stream);
-        launch_pack_blocks(ada_out_w, w_dtype, C, Cs, Cs, 0, C / 32, ROW_NATURAL, K_NATURAL, 1.f, b + l.w_adaout, stream);
         launch_copy_f32(adaln_s_w, w_dtype, reinterpret_cast<float*>(b + l.f_lns_g), Cs, 1.f, stream);
         launch_copy_f32(adaln_g_b, w_dtype, reinterpret_cast<float*>(b + l.f_adag_b), C, 0.f, stream);
         launch_copy_f32(ada_out_b, w_dtype, reinterpret_cast<float*>(b + l.f_adaout_b), C, 0.f, stream);
@@ -197,8 +219,8 @@ int kfh_apb_pack(const void* ln_w, const void* ln_b, const void* q_w, const void
     return check_launch("apb_pack");
 }
 
-size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs) {
-    const ApbLayout l(C, H, Cs);
+size_t kfh_apb_workspace_bytes(int S, int L, int C, int H, int Cs, int arith) {
+    const ApbLayout l(C, H, Cs, arith);
     if (!l.ok || S <= 0 || L <= 0 || L > 8192) return 0;
     return ApbWs(l, S, L).total;
 }
@@ -207,9 +229,9 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
                     const void* blob, const void* residual, void* out, void* workspace,
                     size_t workspace_bytes, int S, int L, int C, int H, int Cs, int apply_norm,
                     int bias_per_sample, int mask_per_sample, int s_per_sample, float eps,
-                    int io_dtype, void* stream_) {
-    const ApbLayout l(C, H, Cs);
-    if (!l.ok) return fail(KFH_EUNSUPPORTED, "apb_forward: C=%d H=%d Cs=%d not supported", C, H, Cs);
+                    int io_dtype, int arith, void* stream_) {
+    const ApbLayout l(C, H, Cs, arith);
+    if (!l.ok) return fail(KFH_EUNSUPPORTED, "apb_forward: C=%d H=%d Cs=%d arith=%d not supported", C, H, Cs, arith);
     if (S <= 0 || L <= 0) return fail(KFH_EINVAL, "apb_forward: bad shape S=%d L=%d", S, L);
     if (L > 8192) return fail(KFH_EUNSUPPORTED, "apb_forward: L=%d > 8192", L);
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "apb_forward: bad io_dtype %d", io_dtype);
@@ -227,30 +249,36 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
     auto f32p = [&](size_t off) { return reinterpret_cast<const float*>(b + off); };
     uint16_t* xn = reinterpret_cast<uint16_t*>(ws + w.xn);
 
-    // 1. normalised input rows (bf16)
+    const int P = l.parts;
+    // with P = 3 a [rows, C] bf16 tensor is three planes `rows * C * 2` bytes apart (split3)
+    auto plane = [&](long long r, int ch) { return P == 3 ? (size_t)r * ch * 2 : (size_t)0; };
+
+    // 1. normalised input rows (bf16, or split fp32)
     if (!apply_norm) {
-        KFH_TRY(launch_rows_norm(a, io_dtype, nullptr, nullptr, xn, rows, C, 0, eps, stream), "rows_norm");
+        KFH_TRY(launch_rows_norm(a, io_dtype, nullptr, nullptr, xn, rows, C, 0, eps, stream, 0, P), "rows_norm");
     } else if (!Cs) {
-        KFH_TRY(launch_rows_norm(a, io_dtype, f32p(l.f_ln_g), f32p(l.f_ln_b), xn, rows, C, 1, eps, stream), "rows_norm");
+        KFH_TRY(launch_rows_norm(a, io_dtype, f32p(l.f_ln_g), f32p(l.f_ln_b), xn, rows, C, 1, eps, stream, 0, P), "rows_norm");
     } else {
         // AdaLN: sigmoid(W_g LN_s(s) + b_g) * LN(a) + W_b LN_s(s)
         const long long srows = s_per_sample ? rows : L;
         uint16_t* an = reinterpret_cast<uint16_t*>(ws + w.an);
         uint16_t* sn = reinterpret_cast<uint16_t*>(ws + w.sn);
         uint16_t* sraw = reinterpret_cast<uint16_t*>(ws + w.sraw);
-        KFH_TRY(launch_rows_norm(a, io_dtype, nullptr, nullptr, an, rows, C, 1, eps, stream), "rows_norm");
-        KFH_TRY(launch_rows_norm(s_cond, io_dtype, f32p(l.f_lns_g), nullptr, sn, srows, Cs, 1, eps, stream), "rows_norm");
-        KFH_TRY(launch_rows_norm(s_cond, io_dtype, nullptr, nullptr, sraw, srows, Cs, 0, eps, stream), "rows_norm");
+        KFH_TRY(launch_rows_norm(a, io_dtype, nullptr, nullptr, an, rows, C, 1, eps, stream, 0, P), "rows_norm");
+        KFH_TRY(launch_rows_norm(s_cond, io_dtype, f32p(l.f_lns_g), nullptr, sn, srows, Cs, 1, eps, stream, 0, P), "rows_norm");
+        KFH_TRY(launch_rows_norm(s_cond, io_dtype, nullptr, nullptr, sraw, srows, Cs, 0, eps, stream, 0, P), "rows_norm");
         LinearArgs p = plain(sn, Cs, L, Cs, b + l.w_adag, C);
         p.rows_a = S; p.a_shared = !s_per_sample;
         p.W2 = b + l.w_adab; p.bias = f32p(l.f_adag_b);
         p.aux = an; p.aux_dtype = KFH_BF16; p.ld_aux = C;
         p.out = xn; p.out_dtype = KFH_BF16; p.ldo = C; p.epi = EPI_ADALN;
+        p.parts = P; p.a_part = plane(srows, Cs); p.w_part = l.wa; p.aux_part = plane(rows, C); p.out_part = plane(rows, C);
         KFH_TRY(launch_linear(p, stream), "linear");
-        // output gate sigmoid(W_ada s + b_ada) on the raw conditioning
+        // output gate sigmoid(W_ada s + b_ada) on the raw conditioning (kept in fp32 in fp32 arithmetic)
         LinearArgs g = plain(sraw, Cs, srows, Cs, b + l.w_adaout, C);
         g.bias = f32p(l.f_adaout_b);
-        g.out = ws + w.gate_out; g.out_dtype = KFH_BF16; g.ldo = C; g.epi = EPI_SIGMOID;
+        g.out = ws + w.gate_out; g.out_dtype = P == 3 ? KFH_F32 : KFH_BF16; g.ldo = C; g.epi = EPI_SIGMOID;
+        g.parts = P; g.a_part = plane(srows, Cs); g.w_part = l.wa;
         KFH_TRY(launch_linear(g, stream), "linear");
     }
 
@@ -258,6 +286,7 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
     {
         LinearArgs p = plain(xn, C, L, C, nullptr, C);
         p.rows_a = S; p.nblk = l.nhb; p.H = H; p.PB = l.PB; p.Dh = l.Dh;
+        p.parts = P; p.a_part = plane(rows, C); p.w_part = l.wh; p.out_part = w.frag;
         p.epi = EPI_FRAG_CH;
         p.W = b + l.wq; p.bias = f32p(l.f_bq); p.bias_scale = kLog2e / sqrtf((float)l.Dh);
         p.out = ws + w.qf;
@@ -279,7 +308,12 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
     fa.qf = ws + w.qf; fa.kf = ws + w.kf; fa.vf = ws + w.vf; fa.gf = ws + w.gf; fa.of = ws + w.of;
     fa.biast = bias_tiles; fa.codes = codes;
     fa.nrows = S; fa.nb = w.nb; fa.H = H; fa.bias_per_row = bias_per_sample ? 1 : 0;
-    if (launch_flash(fa, 32 * l.PB, stream) != 0) return fail(KFH_EUNSUPPORTED, "apb_forward: attention shape");
+    if (P == 3) {
+        fa.q_part = fa.k_part = fa.v_part = fa.g_part = fa.o_part = w.frag;
+        if (launch_flash_split(fa, 32 * l.PB, stream) != 0) return fail(KFH_EUNSUPPORTED, "apb_forward: attention shape");
+    } else if (launch_flash(fa, 32 * l.PB, stream) != 0) {
+        return fail(KFH_EUNSUPPORTED, "apb_forward: attention shape");
+    }
 
     // 4. output projection (+ conditioning gate, + residual)
     {
@@ -287,8 +321,12 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
         p.A = ws + w.of; p.a_frag = 1; p.rows_a = S; p.L = L; p.nb = w.nb; p.K = l.ko * 16;
         p.W = b + l.wo; p.nblk = C / 32; p.Nout = C; p.bias_scale = 1.f;
         p.H = H; p.PB = l.PB; p.Dh = l.Dh;
+        p.parts = P; p.a_part = w.frag; p.w_part = l.wo_bytes;
         p.epi = EPI_RESID;
-        if (cond) { p.gate = reinterpret_cast<const uint16_t*>(ws + w.gate_out); p.ld_gate = C; p.gate_shared = !s_per_sample; }
+        if (cond) {
+            p.gate = reinterpret_cast<const uint16_t*>(ws + w.gate_out); p.ld_gate = C; p.gate_shared = !s_per_sample;
+            p.gate_dtype = P == 3 ? KFH_F32 : KFH_BF16;
+        }
         if (residual) { p.aux = residual; p.aux_dtype = io_dtype; p.ld_aux = C; }
         p.out = out; p.out_dtype = io_dtype; p.ldo = C;
         KFH_TRY(launch_linear(p, stream), "linear");

@@ -49,6 +49,21 @@ __device__ __forceinline__ uint32_t pack_bf16(float a, float b) {
     return __builtin_bit_cast(uint32_t, v);
 }
 
+// x rounded to the nearest bf16 value, as a float
+__device__ __forceinline__ float bf16_round(float x) { return bf16_lo(pack_bf16(x, 0.f)); }
+
+// Three-way split of an fp32 value into bf16-representable parts, x = p[0] + p[1] + p[2] to
+// fp32 accuracy (8 + 8 + 8 significant bits; the two subtractions are exact).  A product of two
+// split operands summed over the part pairs (i, j) with i + j <= 2, each an exact bf16 x bf16
+// product accumulated in fp32, carries fp32 accuracy: this is how the matrix cores run the
+// fp32 ("ieee") arithmetic of the diffusion stack.
+__device__ __forceinline__ void split3(float x, float (&p)[3]) {
+    p[0] = bf16_round(x);
+    const float r = x - p[0];
+    p[1] = bf16_round(r);
+    p[2] = bf16_round(r - p[1]);
+}
+
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
 __device__ __forceinline__ float sigmoidf_fast(float x) {
@@ -98,6 +113,14 @@ __device__ __forceinline__ f32x16 bias_tile_acc(const u32x4& c0, const u32x4& c1
         r[8 + 2 * i + 1] = __uint_as_float(c1[i] & 0xffff0000u);
     }
     return r;
+}
+
+// fp32 tiles of the fp32 arithmetic: [chunk c = 0..3][lane][4], element j of chunk c is
+// accumulator register v = 4c + j (4 KiB per tile, four 16-byte loads per lane)
+constexpr int kBiasTileF32Bytes = 4096;
+__host__ __device__ __forceinline__ int bias_tile_f32_elem(int q32, int k32) {
+    const int v = 4 * (k32 >> 3) + (k32 & 3), lane = q32 + 32 * ((k32 >> 2) & 1);
+    return ((v >> 2) * 64 + lane) * 4 + (v & 3);
 }
 
 // row index inside a 32x32 accumulator block for register v of this lane

@@ -11,9 +11,10 @@ enum : int { K_NATURAL = 0, K_ACC = 1, K_HALF = 2, K_ACC_HEADPAD = 3 };
 constexpr size_t kBlockBytes = 32 * kC * 2;   // one packed 32-row x 128-channel block = 8 KiB
 
 // K: number of k-slots (padded contraction length); ld: row pitch of src in elements
+// part: -1 packs bf16(scale * w); 0..2 packs that part of split3(scale * w) (fp32 arithmetic)
 void launch_pack_blocks(const void* src, int wdtype, int src_rows, int K, int ld, int row0,
                         int nblk, int row_mode, int k_mode, float scale, void* dst,
-                        hipStream_t stream, int kparam = 0);
+                        hipStream_t stream, int kparam = 0, int part = -1);
 void launch_copy_f32(const void* src, int wdtype, float* dst, int n, float fill,
                      hipStream_t stream);
 
@@ -80,8 +81,13 @@ struct FlashArgs {
     int bias_per_row;                 // 0: one bias for all rows, 1: bias batch index = row
     int qgroups, nchunks;             // filled in by launch_flash
     int rowranges, rows_per_range;    // strip kernel: rows are split into ranges per workgroup
+    // fp32 arithmetic (launch_flash_split only): every fragment operand comes as three bf16 parts
+    // (split3), `*_part` bytes apart; the bias tiles are fp32 (bias_tile_f32_elem layout)
+    size_t q_part, k_part, v_part, g_part, o_part;
 };
 int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
+// the same attention in fp32 arithmetic on split operands (flash_split.hip)
+int launch_flash_split(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
 
 void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream);
 // returns 0, or the non-zero status of the attention launch (shape not built, HIP error)
@@ -125,8 +131,10 @@ int launch_parcae_step(const void* z, const void* u, const void* u2, int io_dtyp
 
 // ---- single-track helpers (rows.hip, linear.hip) -------------------------------------------
 // transpose_n > 0: the M = n*n rows are written transposed as an [n, n] grid of rows
+// parts = 3: the result is written as the three split3 planes out[q][M][C] (fp32 arithmetic)
 int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
-                     long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n = 0);
+                     long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n = 0,
+                     int parts = 1);
 // mask element of (row a, key k) is mask[a * mask_stride + k * key_stride]
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
                       long long mask_stride, hipStream_t stream, long long key_stride = 1);
@@ -134,6 +142,9 @@ void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int 
 // L queries in nb blocks, Lk keys (0: = L)
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
                        hipStream_t stream, long long st = 0, long long sq = 0, long long sk = 0, int Lk = 0);
+// the same as fp32 tiles of 4 KiB (bias_tile_f32_elem layout) for the fp32 arithmetic
+void launch_bias_tiles_f32(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
+                           hipStream_t stream, int Lk = 0);
 
 enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS };
 
@@ -151,6 +162,12 @@ struct LinearArgs {
     int epi;
     int H, PB, Dh;                               // heads, 32-blocks per padded head, real head dim
     int out_transposed;                          // EPI_RESID: out / aux row of (a, position) is position * rows_a + a
+    // fp32 arithmetic: parts = 3 — A, W, W2 and every bf16 output (row-major or fragments) are three
+    // split3 planes, `*_part` bytes apart; the EPI_ADALN aux is summed over its three planes;
+    // gate_dtype says how the EPI_RESID gate is stored (a KFH_F32 gate in this mode)
+    int parts;
+    size_t a_part, w_part, out_part, aux_part;
+    int gate_dtype;
 };
 int launch_linear(const LinearArgs& p, hipStream_t stream);
 

@@ -16,30 +16,37 @@
 
 namespace kfh {
 
-template <int EPI, bool AFRAG>
+// PARTS = 3 is the fp32 arithmetic: A, W (and W2) arrive as their three split3 planes and every
+// k-step runs the six part products (i, j), i + j <= 2; bf16 outputs leave as three planes too.
+template <int EPI, bool AFRAG, int PARTS>
 __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, half = lane >> 5;
     // The 4 wavefronts of a workgroup share one 32 x 32 output tile and split K between them in
-    // chunks of 8 k-steps (wavefront w takes chunks w, w+4, ...): these problems have few tiles
+    // chunks of CH k-steps (wavefront w takes chunks w, w+4, ...): these problems have few tiles
     // and long K, so the serial chain of dependent operand loads is what costs.
     __shared__ float red[3][2][64 * 16];
     const int wb = blockIdx.y;
     const int a = blockIdx.x / p.nb, blk = blockIdx.x % p.nb;
     const int ksteps = p.K / 16;
-    const bf16x8* __restrict__ W = static_cast<const bf16x8*>(p.W) + (size_t)wb * ksteps * 64 + lane;
-    const bf16x8* __restrict__ W2 = p.W2 ? static_cast<const bf16x8*>(p.W2) + (size_t)wb * ksteps * 64 + lane : nullptr;
+    const char* Wb = static_cast<const char*>(p.W) + ((size_t)wb * ksteps * 64 + lane) * 16;
+    const char* W2b = p.W2 ? static_cast<const char*>(p.W2) + ((size_t)wb * ksteps * 64 + lane) * 16 : nullptr;
+    auto wfrag = [&](const char* base, int ks, int q) -> bf16x8 {
+        return *reinterpret_cast<const bf16x8*>(base + (size_t)q * p.w_part + (size_t)ks * 1024);
+    };
 
     const int pos = min(blk * 32 + col, p.L - 1);
-    const uint16_t* arow = AFRAG ? nullptr
-                                 : static_cast<const uint16_t*>(p.A) + ((size_t)(p.a_shared ? 0 : a) * p.L + pos) * p.lda + 8 * half;
+    const char* arow = AFRAG ? nullptr
+                             : static_cast<const char*>(p.A) +
+                                   (((size_t)(p.a_shared ? 0 : a) * p.L + pos) * p.lda + 8 * half) * 2;
     const int dks = 2 * p.PB;
-    auto afrag = [&](int ks) -> bf16x8 {
+    auto afrag = [&](int ks, int q) -> bf16x8 {
         if constexpr (AFRAG) {
             const int h = ks / dks, kk = ks % dks;
-            return static_cast<const bf16x8*>(p.A)[((((size_t)a * p.H + h) * p.nb + blk) * dks + kk) * 64 + lane];
+            const size_t u = ((((size_t)a * p.H + h) * p.nb + blk) * dks + kk) * 64 + lane;
+            return *reinterpret_cast<const bf16x8*>(static_cast<const char*>(p.A) + (size_t)q * p.a_part + u * 16);
         } else {
-            return *reinterpret_cast<const bf16x8*>(arow + 16 * ks);
+            return *reinterpret_cast<const bf16x8*>(arow + (size_t)q * p.a_part + 32 * ks);
         }
     };
 
@@ -48,24 +55,33 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
     for (int v = 0; v < 16; ++v) { acc[v] = 0.f; acc2[v] = 0.f; }
     constexpr bool W_IS_A = (EPI == EPI_FRAG_CH);
     constexpr bool TWO = (EPI == EPI_SWIGLU || EPI == EPI_ADALN);
-    // K is walked in chunks of 8 k-steps; the operands of chunk c+1 are
-    // requested before the MFMAs of chunk c, so one memory latency is paid per 8 k-steps at most
-    constexpr int CH = 8;
-    bf16x8 xa[CH], wa[CH], va[CH], xb[CH], wb2[CH], vb[CH];
-    auto load = [&](int c, bf16x8 (&x)[CH], bf16x8 (&w)[CH], bf16x8 (&v)[CH]) {
+    // part pairs (A part, W part) of one k-step, smallest terms first
+    constexpr int NPROD = PARTS == 3 ? 6 : 1;
+    constexpr int PA[6] = {PARTS == 3 ? 2 : 0, PARTS == 3 ? 1 : 0, 0, PARTS == 3 ? 1 : 0, 0, 0};
+    constexpr int PW[6] = {0, PARTS == 3 ? 1 : 0, PARTS == 3 ? 2 : 0, 0, PARTS == 3 ? 1 : 0, 0};
+    // K is walked in chunks of CH k-steps; the operands of chunk c+1 are requested before the
+    // MFMAs of chunk c, so one memory latency is paid per chunk at most
+    constexpr int CH = PARTS == 3 ? 2 : 8;
+    bf16x8 xa[CH][PARTS], wa[CH][PARTS], va[CH][PARTS], xb[CH][PARTS], wb2[CH][PARTS], vb[CH][PARTS];
+    auto load = [&](int c, bf16x8 (&x)[CH][PARTS], bf16x8 (&w)[CH][PARTS], bf16x8 (&v)[CH][PARTS]) {
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
-            x[i] = afrag(c * CH + i);
-            w[i] = W[(size_t)(c * CH + i) * 64];
-            if constexpr (TWO) v[i] = W2[(size_t)(c * CH + i) * 64];
-        }
+        for (int i = 0; i < CH; ++i)
+#pragma unroll
+            for (int q = 0; q < PARTS; ++q) {
+                x[i][q] = afrag(c * CH + i, q);
+                w[i][q] = wfrag(Wb, c * CH + i, q);
+                if constexpr (TWO) v[i][q] = wfrag(W2b, c * CH + i, q);
+            }
     };
-    auto compute = [&](const bf16x8 (&x)[CH], const bf16x8 (&w)[CH], const bf16x8 (&v)[CH]) {
+    auto compute = [&](const bf16x8 (&x)[CH][PARTS], const bf16x8 (&w)[CH][PARTS], const bf16x8 (&v)[CH][PARTS]) {
 #pragma unroll
-        for (int i = 0; i < CH; ++i) {
-            acc = W_IS_A ? mfma32(w[i], x[i], acc) : mfma32(x[i], w[i], acc);
-            if constexpr (TWO) acc2 = mfma32(x[i], v[i], acc2);
-        }
+        for (int i = 0; i < CH; ++i)
+#pragma unroll
+            for (int pr = 0; pr < NPROD; ++pr) {
+                const bf16x8 xq = x[i][PA[pr]], wq = w[i][PW[pr]];
+                acc = W_IS_A ? mfma32(wq, xq, acc) : mfma32(xq, wq, acc);
+                if constexpr (TWO) acc2 = mfma32(xq, v[i][PW[pr]], acc2);
+            }
     };
     const int nch = ksteps / CH;
     const int mine = nch > wave ? (nch - wave + 3) / 4 : 0;          // chunks of this wavefront
@@ -80,11 +96,14 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
         }
     }
     if (wave == 0) {
-        for (int ks = nch * CH; ks < ksteps; ++ks) {      // K not a multiple of 128
-            const bf16x8 x = afrag(ks);
-            const bf16x8 w = W[(size_t)ks * 64];
-            acc = W_IS_A ? mfma32(w, x, acc) : mfma32(x, w, acc);
-            if constexpr (TWO) acc2 = mfma32(x, W2[(size_t)ks * 64], acc2);
+        for (int ks = nch * CH; ks < ksteps; ++ks) {      // K not a multiple of 16 * CH
+#pragma unroll
+            for (int pr = 0; pr < NPROD; ++pr) {
+                const bf16x8 x = afrag(ks, PA[pr]);
+                const bf16x8 w = wfrag(Wb, ks, PW[pr]);
+                acc = W_IS_A ? mfma32(w, x, acc) : mfma32(x, w, acc);
+                if constexpr (TWO) acc2 = mfma32(x, wfrag(W2b, ks, PW[pr]), acc2);
+            }
         }
     }
     // partial sums of wavefronts 1..3 -> LDS -> wavefront 0, which runs the epilogue
@@ -113,20 +132,40 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
                 const int d = 32 * pp + acc_row(v, half);
                 float y = acc[v];
                 if (p.bias && d < p.Dh) y += p.bias[h * p.Dh + d] * p.bias_scale;
-                if (p.sigmoid) y = sigmoidf_fast(y);
+                if (p.sigmoid) y = PARTS == 3 ? 1.0f / (1.0f + exp2f(-kLog2e * y)) : sigmoidf_fast(y);
                 acc[v] = y;
             }
         }
-        bf16x8 f0, f1;
-        acc_to_frags(acc, f0, f1);
-        bf16x8* dst = static_cast<bf16x8*>(p.out) +
-                      ((((size_t)a * p.H + h) * p.nb + blk) * p.PB + pp) * 2 * 64 + lane;
-        dst[0] = f0;
-        dst[64] = f1;
+        const size_t u0 = (((((size_t)a * p.H + h) * p.nb + blk) * p.PB + pp) * 2 * 64 + lane) * 16;
+        if constexpr (PARTS == 1) {
+            bf16x8 f0, f1;
+            acc_to_frags(acc, f0, f1);
+            bf16x8* dst = reinterpret_cast<bf16x8*>(static_cast<char*>(p.out) + u0);
+            dst[0] = f0;
+            dst[64] = f1;
+        } else {
+            f32x16 part[PARTS];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float sp[3];
+                split3(acc[v], sp);
+#pragma unroll
+                for (int q = 0; q < PARTS; ++q) part[q][v] = sp[q];
+            }
+#pragma unroll
+            for (int q = 0; q < PARTS; ++q) {
+                bf16x8 f0, f1;
+                acc_to_frags(part[q], f0, f1);
+                bf16x8* dst = reinterpret_cast<bf16x8*>(static_cast<char*>(p.out) + (size_t)q * p.out_part + u0);
+                dst[0] = f0;
+                dst[64] = f1;
+            }
+        }
     } else {
         const int c = 32 * wb + col;
         if (c >= p.Nout) return;
         const float bc = p.bias ? p.bias[c] : 0.f;
+        auto sig = [&](float x) { return PARTS == 3 ? 1.0f / (1.0f + exp2f(-kLog2e * x)) : sigmoidf_fast(x); };
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int ps = blk * 32 + acc_row(v, half);
@@ -138,21 +177,38 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
             }
             const size_t r_gate = (size_t)(p.gate_shared ? 0 : a) * p.L + ps;
             float y = acc[v] + bc;
-            if constexpr (EPI == EPI_SIGMOID) y = sigmoidf_fast(y);
-            if constexpr (EPI == EPI_SWIGLU) y = acc[v] * sigmoidf_fast(acc[v]) * acc2[v];
+            if constexpr (EPI == EPI_SIGMOID) y = sig(y);
+            if constexpr (EPI == EPI_SWIGLU) y = acc[v] * sig(acc[v]) * acc2[v];
             if constexpr (EPI == EPI_ADALN) {
-                const float ax = bf16_lo(static_cast<const uint16_t*>(p.aux)[r_aux * p.ld_aux + c]);
-                y = sigmoidf_fast(y) * ax + acc2[v];
+                const char* ap = static_cast<const char*>(p.aux) + (r_aux * p.ld_aux + c) * 2;
+                float ax = bf16_lo(*reinterpret_cast<const uint16_t*>(ap));
+                if constexpr (PARTS == 3)
+                    ax = (bf16_lo(*reinterpret_cast<const uint16_t*>(ap + 2 * p.aux_part)) +
+                          bf16_lo(*reinterpret_cast<const uint16_t*>(ap + p.aux_part))) + ax;
+                y = sig(y) * ax + acc2[v];
             }
             if constexpr (EPI == EPI_RESID) {
-                if (p.gate) y *= bf16_lo(p.gate[r_gate * p.ld_gate + c]);
+                if (p.gate) {
+                    y *= p.gate_dtype == KFH_F32 ? reinterpret_cast<const float*>(p.gate)[r_gate * p.ld_gate + c]
+                                                 : bf16_lo(p.gate[r_gate * p.ld_gate + c]);
+                }
                 if (p.aux) {
                     y += p.aux_dtype == KFH_F32 ? static_cast<const float*>(p.aux)[r_aux * p.ld_aux + c]
                                                 : bf16_lo(static_cast<const uint16_t*>(p.aux)[r_aux * p.ld_aux + c]);
                 }
             }
-            if (p.out_dtype == KFH_F32) static_cast<float*>(p.out)[r * p.ldo + c] = y;
-            else static_cast<uint16_t*>(p.out)[r * p.ldo + c] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
+            if (p.out_dtype == KFH_F32) {
+                static_cast<float*>(p.out)[r * p.ldo + c] = y;
+            } else if constexpr (PARTS == 1) {
+                static_cast<uint16_t*>(p.out)[r * p.ldo + c] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
+            } else {
+                float sp[3];
+                split3(y, sp);
+#pragma unroll
+                for (int q = 0; q < PARTS; ++q)
+                    *reinterpret_cast<uint16_t*>(static_cast<char*>(p.out) + (size_t)q * p.out_part + (r * p.ldo + c) * 2) =
+                        (uint16_t)(pack_bf16(sp[q], 0.f) & 0xffffu);
+            }
         }
     }
 }
@@ -160,15 +216,27 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
 int launch_linear(const LinearArgs& p, hipStream_t stream) {
     if (p.K % 16 || p.nb <= 0 || p.rows_a <= 0) return -1;
     dim3 grid((unsigned)(p.rows_a * p.nb), (unsigned)p.nblk), block(256);
-#define KFH_LIN(E, F) hipLaunchKernelGGL((linear_kernel<E, F>), grid, block, 0, stream, p)
+#define KFH_LIN(E, F, P) hipLaunchKernelGGL((linear_kernel<E, F, P>), grid, block, 0, stream, p)
+    if (p.parts == 3) {          // fp32 arithmetic on split operands (pair-bias attention only)
+        switch (p.epi) {
+            case EPI_SIGMOID: KFH_LIN(EPI_SIGMOID, false, 3); break;
+            case EPI_ADALN: KFH_LIN(EPI_ADALN, false, 3); break;
+            case EPI_RESID: if (p.a_frag) KFH_LIN(EPI_RESID, true, 3); else return -1; break;
+            case EPI_FRAG_CH: KFH_LIN(EPI_FRAG_CH, false, 3); break;
+            case EPI_FRAG_POS: KFH_LIN(EPI_FRAG_POS, false, 3); break;
+            default: return -1;
+        }
+        return 0;
+    }
+    if (p.parts != 0 && p.parts != 1) return -1;
     switch (p.epi) {
-        case EPI_STORE: if (p.a_frag) KFH_LIN(EPI_STORE, true); else KFH_LIN(EPI_STORE, false); break;
-        case EPI_SIGMOID: KFH_LIN(EPI_SIGMOID, false); break;
-        case EPI_SWIGLU: KFH_LIN(EPI_SWIGLU, false); break;
-        case EPI_ADALN: KFH_LIN(EPI_ADALN, false); break;
-        case EPI_RESID: if (p.a_frag) KFH_LIN(EPI_RESID, true); else KFH_LIN(EPI_RESID, false); break;
-        case EPI_FRAG_CH: KFH_LIN(EPI_FRAG_CH, false); break;
-        case EPI_FRAG_POS: KFH_LIN(EPI_FRAG_POS, false); break;
+        case EPI_STORE: if (p.a_frag) KFH_LIN(EPI_STORE, true, 1); else KFH_LIN(EPI_STORE, false, 1); break;
+        case EPI_SIGMOID: KFH_LIN(EPI_SIGMOID, false, 1); break;
+        case EPI_SWIGLU: KFH_LIN(EPI_SWIGLU, false, 1); break;
+        case EPI_ADALN: KFH_LIN(EPI_ADALN, false, 1); break;
+        case EPI_RESID: if (p.a_frag) KFH_LIN(EPI_RESID, true, 1); else KFH_LIN(EPI_RESID, false, 1); break;
+        case EPI_FRAG_CH: KFH_LIN(EPI_FRAG_CH, false, 1); break;
+        case EPI_FRAG_POS: KFH_LIN(EPI_FRAG_POS, false, 1); break;
         default: return -1;
     }
 #undef KFH_LIN

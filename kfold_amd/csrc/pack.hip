@@ -38,7 +38,7 @@ __device__ __forceinline__ int pack_k(int mode, int K, int ks, int half, int e, 
 template <int WT>
 __global__ void pack_blocks_kernel(const void* __restrict__ src, int src_rows, int K, int ld,
                                    int row0, int nblk, int row_mode, int k_mode, int kparam,
-                                   float scale, uint16_t* __restrict__ dst) {
+                                   float scale, uint16_t* __restrict__ dst, int part) {
     const int ksteps = K / 16;
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;      // (block, ks, lane)
     if (idx >= nblk * ksteps * 64) return;
@@ -61,6 +61,11 @@ __global__ void pack_blocks_kernel(const void* __restrict__ src, int src_rows, i
                 else x = bf16_lo(static_cast<const uint16_t*>(src)[off]);
             }
             v[u] = x * scale;
+            if (part >= 0) {
+                float sp[3];
+                split3(v[u], sp);
+                v[u] = sp[part];
+            }
         }
         w[e >> 1] = pack_bf16(v[0], v[1]);
     }
@@ -97,17 +102,17 @@ void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream) {
 
 void launch_pack_blocks(const void* src, int wdtype, int src_rows, int K, int ld, int row0,
                         int nblk, int row_mode, int k_mode, float scale, void* dst,
-                        hipStream_t stream, int kparam) {
+                        hipStream_t stream, int kparam, int part) {
     const int total = nblk * (K / 16) * 64;
     const int threads = 256, blocks = (total + threads - 1) / threads;
     if (wdtype == KFH_F32)
         hipLaunchKernelGGL(pack_blocks_kernel<KFH_F32>, dim3(blocks), dim3(threads), 0, stream, src,
                            src_rows, K, ld, row0, nblk, row_mode, k_mode, kparam, scale,
-                           static_cast<uint16_t*>(dst));
+                           static_cast<uint16_t*>(dst), part);
     else
         hipLaunchKernelGGL(pack_blocks_kernel<KFH_BF16>, dim3(blocks), dim3(threads), 0, stream, src,
                            src_rows, K, ld, row0, nblk, row_mode, k_mode, kparam, scale,
-                           static_cast<uint16_t*>(dst));
+                           static_cast<uint16_t*>(dst), part);
 }
 
 void launch_copy_f32(const void* src, int wdtype, float* dst, int n, float fill,

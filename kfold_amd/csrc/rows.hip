@@ -15,7 +15,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 // gamma / beta may be null (1 / 0).  C is even, at most 2048.  With tn > 0 the rows are the
 // positions (i, j) of a [tn, tn] grid and are written transposed: r = i * tn + j -> r' = j * tn + i.
 // (reference: model/primitives/normalization.py:61-91 — fp32 statistics, biased variance)
-template <int IO>
+// PARTS = 3: the fp32 result is written as its three split3 planes, plane q at out + q * M * C.
+template <int IO, int PARTS = 1>
 __global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__ x,
                                                         const float* __restrict__ gamma,
                                                         const float* __restrict__ beta,
@@ -66,15 +67,35 @@ __global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__
             if (gamma) { u *= gamma[c]; v *= gamma[c + 1]; }
             if (beta) { u += beta[c]; v += beta[c + 1]; }
         }
-        *reinterpret_cast<uint32_t*>(out + (size_t)ro * C + c) = pack_bf16(u, v);
+        if constexpr (PARTS == 1) {
+            *reinterpret_cast<uint32_t*>(out + (size_t)ro * C + c) = pack_bf16(u, v);
+        } else {
+            float pu[3], pv[3];
+            split3(u, pu);
+            split3(v, pv);
+#pragma unroll
+            for (int q = 0; q < PARTS; ++q)
+                *reinterpret_cast<uint32_t*>(out + (size_t)q * M * C + (size_t)ro * C + c) = pack_bf16(pu[q], pv[q]);
+        }
     }
 }
 
 int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
-                     long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n) {
+                     long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n,
+                     int parts) {
     if (C % 2 || C > 2048 || C <= 0) return -1;
     if (transpose_n > 0 && (long long)transpose_n * transpose_n != M) return -1;
+    if (parts != 1 && parts != 3) return -1;
     dim3 grid((unsigned)((M + 3) / 4)), block(256);
+    if (parts == 3) {
+        if (io_dtype == KFH_F32)
+            hipLaunchKernelGGL((rows_norm_kernel<KFH_F32, 3>), grid, block, 0, stream, x, gamma, beta, out, M, C,
+                               normalize, eps, transpose_n);
+        else
+            hipLaunchKernelGGL((rows_norm_kernel<KFH_BF16, 3>), grid, block, 0, stream, x, gamma, beta, out, M, C,
+                               normalize, eps, transpose_n);
+        return 0;
+    }
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(rows_norm_kernel<KFH_F32>, grid, block, 0, stream, x, gamma, beta, out, M, C,
                            normalize, eps, transpose_n);
@@ -149,6 +170,45 @@ void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nba
     else
         hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, Lq, Lk, nbq,
                            nbk, st, sq, sk);
+}
+
+// Dense pair bias -> log2(e)-scaled fp32 tiles (bias_tile_f32_elem layout): one thread writes the
+// 4 keys of one (tile, chunk, lane) slot.  Source [nbatch][H][Lq][Lk] contiguous.
+template <int IO>
+__global__ void bias_tiles_f32_kernel(const void* __restrict__ dense, float* __restrict__ tiles,
+                                      long long total, int Lq, int Lk, int nbq, int nbk) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;      // 16-byte slot
+    if (i >= total) return;
+    const int lane = (int)(i & 63), c = (int)((i >> 6) & 3);
+    long long t = i >> 8;
+    const int kb = (int)(t % nbk); t /= nbk;
+    const int qb = (int)(t % nbq); t /= nbq;        // t = batch * H + h
+    const int q = qb * 32 + (lane & 31);
+    f32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int k = kb * 32 + acc_row(4 * c + e, lane >> 5);
+        float x = 0.f;
+        if (q < Lq && k < Lk) {
+            const size_t off = ((size_t)t * Lq + q) * Lk + k;
+            if constexpr (IO == KFH_F32) x = static_cast<const float*>(dense)[off];
+            else x = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
+        }
+        o[e] = x * kLog2e;
+    }
+    reinterpret_cast<f32x4*>(tiles)[i] = o;
+}
+
+void launch_bias_tiles_f32(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
+                           hipStream_t stream, int Lk) {
+    if (Lk <= 0) Lk = L;
+    const int nbk = (Lk + 31) / 32;
+    const long long total = (long long)nbatch * H * nb * nbk * 256;
+    dim3 grid((unsigned)((total + 255) / 256)), block(256);
+    if (io_dtype == KFH_F32)
+        hipLaunchKernelGGL(bias_tiles_f32_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, L, Lk, nb, nbk);
+    else
+        hipLaunchKernelGGL(bias_tiles_f32_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, L, Lk, nb, nbk);
 }
 
 }  // namespace kfh

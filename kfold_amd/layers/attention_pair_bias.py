@@ -9,6 +9,13 @@
 
 ``CrossAttentionPairBias`` mirrors the local-window attention of the atom transformer
 (:161-260): Lq queries against Lk keys per window, one bias and key mask per window.
+
+Arithmetic.  The reference runs its trunk and confidence head under bf16 autocast
+(inference/runner.py:565-571) and its diffusion stack outside it, on fp32 tensors with full
+fp32 dot products (model/model.py:419, kernels/triton/attention_pair_bias/dispatch.py:439,453).
+The modules here follow that: ``arith = "auto"`` (the default) selects the library's fp32
+arithmetic (``KFH_ARITH_F32``) for a diffusion call site when the activations are fp32 and
+autocast is off, and bf16 arithmetic everywhere else; ``"bf16"`` / ``"f32"`` force one.
 """
 
 from __future__ import annotations
@@ -52,6 +59,20 @@ def norm_eps(module: nn.Module) -> float:
     return module.layernorm_a.eps if hasattr(module, "layernorm_a") else 1e-5
 
 
+def select_arith(module: nn.Module, x: torch.Tensor) -> int:
+    mode = getattr(module, "arith", "auto")
+    if mode == "f32":
+        return ops.KFH_ARITH_F32
+    if mode == "bf16":
+        return ops.KFH_ARITH_BF16
+    if mode != "auto":
+        raise ValueError(f"arith must be 'auto', 'bf16' or 'f32', got {mode!r}")
+    diffusion = str(getattr(module, "call_site", "diffusion_local")).startswith("diffusion")
+    if diffusion and x.dtype == torch.float32 and not torch.is_autocast_enabled():
+        return ops.KFH_ARITH_F32
+    return ops.KFH_ARITH_BF16
+
+
 def _flatten(t: torch.Tensor, keep: int, lead: torch.Size):
     """Flatten the leading dims of ``t`` (which broadcast against ``lead``) to 1 or prod(lead)."""
     tl = t.shape[:t.dim() - keep]
@@ -68,9 +89,11 @@ def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
         raise NotImplementedError("hip pair-bias attention: gate / output projection biases")
     params = _parameters(module)
     C, H, Cs = module.channel_a, module.num_heads, _cond_channels(module)
-    key = cache_key(tuple(params.values()), a, torch.bfloat16)
+    arith = select_arith(module, a)
+    key = cache_key(tuple(params.values()), a,
+                    torch.float32 if arith == ops.KFH_ARITH_F32 else torch.bfloat16)
     blob = cached_blob(module, "_hip_apb_cache", key,
-                       lambda: ops.apb_pack(C, H, Cs, device=a.device, **params))
+                       lambda: ops.apb_pack(C, H, Cs, device=a.device, arith=arith, **params))
     lead = a.shape[:-2]
     io = a if a.dtype in (torch.bfloat16, torch.float32) else a.float()
     af = io.reshape((-1,) + a.shape[-2:])
@@ -79,20 +102,51 @@ def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
     sf = None
     if s is not None and apply_norm and Cs:
         sf, _ = _flatten(s, 2, lead)
-    tiles = ops.bias_tiles_from_dense(pb)
+    tiles = ops.bias_tiles_from_dense(pb, arith)
     out = ops.apb_forward(af, sf, tiles, mk, blob, H, Cs, apply_norm, per_sample and af.shape[0] > 1,
-                          eps=norm_eps(module))
+                          eps=norm_eps(module), arith=arith)
     return out.reshape(a.shape).to(a.dtype)
+
+
+def _run_cross(module, x_q, x_k, pair_bias, mask) -> torch.Tensor:
+    """Already normalised queries x_q [*, Lq, C] against keys x_k [*, Lk, C]: q/k/v/gate/output
+    projections and the attention only (the caller has normalised and applies its own
+    conditioning gate afterwards, attention_pair_bias.py:241-262 of the reference)."""
+    check_inference(x_q, "cross attention with pair bias")
+    check_inf(module)
+    if module.linear_g.bias is not None or module.linear_out.bias is not None:
+        raise NotImplementedError("hip cross attention: gate / output projection biases")
+    w = dict(q_w=module.linear_q.weight, q_b=module.linear_q.bias, k_w=module.linear_k.weight,
+             v_w=module.linear_v.weight, g_w=module.linear_g.weight, o_w=module.linear_out.weight)
+    arith = select_arith(module, x_q)
+    C, H = module.channel_a, module.num_heads
+    key = cache_key(tuple(w.values()), x_q, torch.float32 if arith == ops.KFH_ARITH_F32 else torch.bfloat16)
+    blob = cached_blob(module, "_hip_cross_functional_cache", key,
+                       lambda: ops.cross_apb_pack(C, H, 0, x_q.device, arith=arith, **w))
+    lead = x_q.shape[:-2]
+    Lq = x_q.shape[-2]
+    io = x_q if x_q.dtype in (torch.bfloat16, torch.float32) else x_q.float()
+
+    def flat(t, keep):
+        full = torch.broadcast_to(t, tuple(lead) + t.shape[t.dim() - keep:])
+        return full.reshape((-1,) + t.shape[t.dim() - keep:])
+
+    out = ops.cross_apb_forward(io.reshape(-1, Lq, C), flat(x_k, 2), None, None, flat(pair_bias, 3),
+                                flat(mask, 1), blob, H, 0, apply_norm=False, arith=arith)
+    return out.reshape(x_q.shape).to(x_q.dtype)
 
 
 @torch.compiler.disable
 def hip_attention_pair_bias(module: nn.Module, x_q: torch.Tensor, x_k: torch.Tensor,
                             pair_bias: torch.Tensor, mask: torch.Tensor, *,
                             call_site: str = "confidence") -> torch.Tensor:
-    """x_q, x_k [*, L, C] normalised (must be the same tensor), pair_bias broadcastable to
-    [*, H, L, L], mask broadcastable to [*, L]."""
-    if x_q is not x_k and (x_q.shape != x_k.shape or x_q.data_ptr() != x_k.data_ptr()):
-        raise NotImplementedError("hip pair-bias attention is built for self attention only")
+    """x_q [*, Lq, C], x_k [*, Lk, C] normalised, pair_bias broadcastable to [*, H, Lq, Lk], mask
+    broadcastable to [*, Lk] (the signature of model/primitives/attention.py:28-37).  The same
+    tensor on both sides is self attention; different tensors are the local windows of
+    ``CrossAttentionPairBias`` (call site "diffusion_local")."""
+    if x_q is not x_k and (x_q.shape != x_k.shape or x_q.data_ptr() != x_k.data_ptr()
+                           or x_q.stride() != x_k.stride()):
+        return _run_cross(module, x_q, x_k, pair_bias, mask)
     return _run(module, x_q, None, pair_bias, mask, apply_norm=False)
 
 
@@ -109,13 +163,14 @@ class AdaLN(nn.Module):
 
 class SelfAttentionPairBias(nn.Module):
     def __init__(self, channel_a: int, num_heads: int, channel_s: int | None, call_site: str,
-                 inf: float = 1e9, kernel_backend: str = "hip") -> None:
+                 inf: float = 1e9, kernel_backend: str = "hip", arith: str = "auto") -> None:
         super().__init__()
         if kernel_backend != "hip":
             raise ValueError(
                 f"kfold_amd implements kernel_backend='hip' only, got {kernel_backend!r}")
         if call_site not in {"diffusion_global", "confidence"}:
             raise ValueError(f"Unsupported self APB call site: {call_site!r}")
+        self.arith = arith
         assert channel_a % num_heads == 0
         self.use_single_conditioning = channel_s is not None
         self.call_site = call_site
@@ -154,11 +209,13 @@ class CrossAttentionPairBias(nn.Module):
     ``adaln_a_k`` + ``linear_ada_out``) and ``forward(a_q, a_k, s_q, s_k, pair_bias, mask)``."""
 
     def __init__(self, channel_a: int, num_heads: int, channel_s: int | None, inf: float = 1e9,
-                 kernel_backend: str = "hip") -> None:
+                 kernel_backend: str = "hip", arith: str = "auto") -> None:
         super().__init__()
         if kernel_backend != "hip":
             raise ValueError(f"kfold_amd implements kernel_backend='hip' only, got {kernel_backend!r}")
         assert channel_a % num_heads == 0
+        self.arith = arith
+        self.call_site = "diffusion_local"
         self.use_single_conditioning = channel_s is not None
         self.channel_a = channel_a
         self.channel_s = channel_s
@@ -211,8 +268,11 @@ class CrossAttentionPairBias(nn.Module):
             raise NotImplementedError("hip cross attention: gate / output projection biases")
         w = self._weights()
         cs = self.channel_s or 0
-        blob = cached_blob(self, "_hip_cross_cache", cache_key(tuple(w.values()), a_q, torch.bfloat16),
-                           lambda: ops.cross_apb_pack(self.channel_a, self.num_heads, cs, a_q.device, **w))
+        arith = select_arith(self, a_q)
+        key = cache_key(tuple(w.values()), a_q, torch.float32 if arith == ops.KFH_ARITH_F32 else torch.bfloat16)
+        blob = cached_blob(self, "_hip_cross_cache", key,
+                           lambda: ops.cross_apb_pack(self.channel_a, self.num_heads, cs, a_q.device,
+                                                      arith=arith, **w))
         lead = a_q.shape[:-2]
         Lq, Lk = a_q.shape[-2], a_k.shape[-2]
         io = a_q if a_q.dtype in (torch.bfloat16, torch.float32) else a_q.float()
@@ -224,5 +284,6 @@ class CrossAttentionPairBias(nn.Module):
         eps = (self.adaln_a_q.layernorm_a.eps if self.use_single_conditioning else self.layernorm_a_q.eps)
         out = ops.cross_apb_forward(io.reshape(-1, Lq, self.channel_a), flat(a_k, 2),
                                     None if s_q is None else flat(s_q, 2), None if s_k is None else flat(s_k, 2),
-                                    flat(pair_bias, 3), flat(mask, 1), blob, self.num_heads, cs, eps=eps)
+                                    flat(pair_bias, 3), flat(mask, 1), blob, self.num_heads, cs, eps=eps,
+                                    arith=arith)
         return out.reshape(a_q.shape).to(a_q.dtype)

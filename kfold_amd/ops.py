@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from . import _lib
-from ._lib import KFH_BF16, KFH_F32, KFH_INCOMING, KFH_OUTGOING, check
+from ._lib import KFH_ARITH_BF16, KFH_ARITH_F32, KFH_BF16, KFH_F32, KFH_INCOMING, KFH_OUTGOING, check
 
 _IO_DTYPES = {torch.bfloat16: KFH_BF16, torch.float32: KFH_F32}
 
@@ -74,7 +74,7 @@ def _workspace(given: torch.Tensor | None, need: int, dev: torch.device) -> torc
 def workspace_bytes(op: str, **shape) -> int:
     """Bytes of scratch memory a forward call needs (0: shape not supported): ``trimul`` (N, C),
     ``triattn`` (N, C, heads), ``transition`` (rows, C, expansion), ``apb`` (S, L, C, heads,
-    cond_channels), ``cross_apb`` (W, Lq, Lk, C, heads, cond_channels).  Needs no GPU."""
+    cond_channels, arith), ``cross_apb`` (W, Lq, Lk, C, heads, cond_channels, arith).  Needs no GPU."""
     L = _lib.lib()
     g = shape.__getitem__
     if op == "trimul":
@@ -84,10 +84,11 @@ def workspace_bytes(op: str, **shape) -> int:
     if op == "transition":
         return L.kfh_transition_workspace_bytes(g("rows"), g("C"), g("expansion"))
     if op == "apb":
-        return L.kfh_apb_workspace_bytes(g("S"), g("L"), g("C"), g("heads"), shape.get("cond_channels", 0))
+        return L.kfh_apb_workspace_bytes(g("S"), g("L"), g("C"), g("heads"), shape.get("cond_channels", 0),
+                                         shape.get("arith", KFH_ARITH_BF16))
     if op == "cross_apb":
         return L.kfh_cross_apb_workspace_bytes(g("W"), g("Lq"), g("Lk"), g("C"), g("heads"),
-                                               shape.get("cond_channels", 0))
+                                               shape.get("cond_channels", 0), shape.get("arith", KFH_ARITH_BF16))
     raise ValueError(f"unknown op {op!r}")
 
 
@@ -266,8 +267,9 @@ def transition_forward(x: torch.Tensor, blob: torch.Tensor, expansion: int, eps:
 # ---------------------------------------------------------------------------------------
 # pair bias tiles and pair-bias attention
 # ---------------------------------------------------------------------------------------
-def bias_tiles_from_dense(pair_bias: torch.Tensor) -> torch.Tensor:
-    """Dense pair bias [nbatch, H, L, L] -> the attention kernel's fp32 tiles (flat uint8)."""
+def bias_tiles_from_dense(pair_bias: torch.Tensor, arith: int = KFH_ARITH_BF16) -> torch.Tensor:
+    """Dense pair bias [nbatch, H, L, L] -> the attention kernel's bias tiles (flat uint8): bf16
+    tiles, or fp32 tiles for ``arith=KFH_ARITH_F32``."""
     dev = _require_cuda(pair_bias)
     nbatch, H, Lq, Lk = pair_bias.shape
     if Lq != Lk:
@@ -276,10 +278,10 @@ def bias_tiles_from_dense(pair_bias: torch.Tensor) -> torch.Tensor:
     if pb.dtype not in _IO_DTYPES:
         pb = pb.float()
     L = _lib.lib()
-    tiles = torch.empty(L.kfh_bias_tiles_bytes(nbatch, H, Lq), dtype=torch.uint8, device=dev)
+    tiles = torch.empty(L.kfh_bias_tiles_bytes(nbatch, H, Lq, arith), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(L.kfh_bias_tiles_from_dense(pb.data_ptr(), _io_dtype(pb), tiles.data_ptr(), nbatch, H, Lq,
-                                          _stream(dev)))
+                                          arith, _stream(dev)))
     return tiles
 
 
@@ -303,7 +305,7 @@ def pair_bias_project(z: torch.Tensor, blob: torch.Tensor, heads: int, eps: floa
     assert N == N2
     zc = z.contiguous()
     L = _lib.lib()
-    tiles = torch.empty(L.kfh_bias_tiles_bytes(B, heads, N), dtype=torch.uint8, device=dev)
+    tiles = torch.empty(L.kfh_bias_tiles_bytes(B, heads, N, KFH_ARITH_BF16), dtype=torch.uint8, device=dev)
     with torch.cuda.device(dev):
         check(L.kfh_pair_bias_project(zc.data_ptr(), blob.data_ptr(), tiles.data_ptr(), B, N, C, heads,
                                       float(eps), _io_dtype(zc), _stream(dev)))
@@ -312,9 +314,9 @@ def pair_bias_project(z: torch.Tensor, blob: torch.Tensor, heads: int, eps: floa
 
 def apb_pack(C: int, H: int, Cs: int, *, ln_w=None, ln_b=None, q_w, q_b, k_w, v_w, g_w, o_w,
              adaln_s_w=None, adaln_g_w=None, adaln_g_b=None, adaln_bias_w=None, ada_out_w=None,
-             ada_out_b=None, device: torch.device) -> torch.Tensor:
+             ada_out_b=None, device: torch.device, arith: int = KFH_ARITH_BF16) -> torch.Tensor:
     L = _lib.lib()
-    nbytes = L.kfh_apb_packed_bytes(C, H, Cs)
+    nbytes = L.kfh_apb_packed_bytes(C, H, Cs, arith)
     if nbytes == 0:
         raise NotImplementedError(
             f"hip pair-bias attention: C={C}, H={H}, Cs={Cs} unsupported "
@@ -323,16 +325,18 @@ def apb_pack(C: int, H: int, Cs: int, *, ln_w=None, ln_b=None, q_w, q_b, k_w, v_
                       adaln_g_b, adaln_bias_w, ada_out_w, ada_out_b)
     blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
-        check(L.kfh_apb_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, Cs, blob.data_ptr(), _stream(device)))
+        check(L.kfh_apb_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, Cs, arith, blob.data_ptr(), _stream(device)))
     return blob
 
 
 def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tensor, mask: torch.Tensor,
                 blob: torch.Tensor, heads: int, cond_channels: int, apply_norm: bool,
                 bias_per_sample: bool, eps: float = 1e-5, residual: torch.Tensor | None = None,
-                out: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+                out: torch.Tensor | None = None, workspace: torch.Tensor | None = None,
+                arith: int = KFH_ARITH_BF16) -> torch.Tensor:
     """a [S, L, C]; s_cond [S or 1, L, Cs] or None; mask [S or 1, L]; tiles from the calls above;
-    ``workspace`` as in ``trimul_forward`` (``workspace_bytes("apb", S=, L=, C=, heads=, cond_channels=)``)."""
+    ``workspace`` as in ``trimul_forward`` (``workspace_bytes("apb", S=, L=, C=, heads=, cond_channels=,
+    arith=)``).  ``arith``: the arithmetic the blob and the tiles were made for."""
     dev = _require_cuda(a, s_cond, tiles, mask, blob, residual, out)
     S, Lq, C = a.shape
     ac = a.contiguous()
@@ -354,7 +358,7 @@ def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tenso
                                  or not residual.is_contiguous()):
         raise ValueError("residual must be contiguous with the shape and dtype of a")
     L = _lib.lib()
-    ws_bytes = L.kfh_apb_workspace_bytes(S, Lq, C, heads, cond_channels)
+    ws_bytes = L.kfh_apb_workspace_bytes(S, Lq, C, heads, cond_channels, arith)
     if ws_bytes == 0:
         raise NotImplementedError(f"hip pair-bias attention: unsupported shape S={S} L={Lq} C={C} H={heads}")
     ws = _workspace(workspace, ws_bytes, dev)
@@ -364,7 +368,7 @@ def apb_forward(a: torch.Tensor, s_cond: torch.Tensor | None, tiles: torch.Tenso
                                 cond_channels, 1 if apply_norm else 0, 1 if bias_per_sample else 0,
                                 1 if m8.shape[0] == S and S > 1 else 0,
                                 1 if sc is not None and sc.shape[0] == S and S > 1 else 0,
-                                float(eps), _io_dtype(ac), _stream(dev)))
+                                float(eps), _io_dtype(ac), arith, _stream(dev)))
     return out
 
 
@@ -417,24 +421,29 @@ _CROSS_ORDER = ("lnq_w", "lnq_b", "lnk_w", "lnk_b", "q_w", "q_b", "k_w", "v_w", 
                 "ada_out_w", "ada_out_b")
 
 
-def cross_apb_pack(C: int, H: int, Cs: int, device: torch.device, **weights) -> torch.Tensor:
+def cross_apb_pack(C: int, H: int, Cs: int, device: torch.device, arith: int = KFH_ARITH_BF16,
+                   **weights) -> torch.Tensor:
     L = _lib.lib()
-    nbytes = L.kfh_cross_apb_packed_bytes(C, H, Cs)
+    nbytes = L.kfh_cross_apb_packed_bytes(C, H, Cs, arith)
     if nbytes == 0:
         raise NotImplementedError(f"hip cross attention: C={C}, H={H}, Cs={Cs} unsupported")
     ws = _weights_f32(device, *[weights.get(k) for k in _CROSS_ORDER])
     blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
-        check(L.kfh_cross_apb_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, Cs, blob.data_ptr(), _stream(device)))
+        check(L.kfh_cross_apb_pack(*[_ptr(t) for t in ws], KFH_F32, C, H, Cs, arith, blob.data_ptr(),
+                                   _stream(device)))
     return blob
 
 
 def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias: torch.Tensor, mask: torch.Tensor,
                       blob: torch.Tensor, heads: int, cond_channels: int, eps: float = 1e-5,
                       residual: torch.Tensor | None = None, out: torch.Tensor | None = None,
-                      workspace: torch.Tensor | None = None) -> torch.Tensor:
+                      workspace: torch.Tensor | None = None, apply_norm: bool = True,
+                      arith: int = KFH_ARITH_BF16) -> torch.Tensor:
     """a_q [W, Lq, C], a_k [W, Lk, C], s_q / s_k [W, L., Cs] or None, pair_bias [W, H, Lq, Lk], mask [W, Lk];
-    ``workspace`` as in ``trimul_forward`` (``workspace_bytes("cross_apb", W=, Lq=, Lk=, C=, heads=, cond_channels=)``)."""
+    ``workspace`` as in ``trimul_forward`` (``workspace_bytes("cross_apb", W=, Lq=, Lk=, C=, heads=,
+    cond_channels=, arith=)``).  ``apply_norm=False``: a_q / a_k are already normalised (the functional
+    entry); then no conditioning is applied either."""
     dev = _require_cuda(a_q, a_k, s_q, s_k, pair_bias, mask, blob, residual, out)
     W, Lq, C = a_q.shape
     Lk = a_k.shape[1]
@@ -446,7 +455,7 @@ def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias:
         pb = pb.float()
     m8 = _mask_bytes(mask, mask.shape)
     sq = sk = None
-    if cond_channels:
+    if cond_channels and apply_norm:
         sq, sk = s_q.contiguous().to(aq.dtype), s_k.contiguous().to(aq.dtype)
         if sq.shape != (W, Lq, cond_channels) or sk.shape != (W, Lk, cond_channels):
             raise ValueError("cross attention: conditioning shapes do not match")
@@ -458,7 +467,7 @@ def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias:
                                  or not residual.is_contiguous()):
         raise ValueError("residual must be contiguous with the shape and dtype of a_q")
     L = _lib.lib()
-    ws_bytes = L.kfh_cross_apb_workspace_bytes(W, Lq, Lk, C, heads, cond_channels)
+    ws_bytes = L.kfh_cross_apb_workspace_bytes(W, Lq, Lk, C, heads, cond_channels, arith)
     if ws_bytes == 0:
         raise NotImplementedError(f"hip cross attention: unsupported shape W={W} Lq={Lq} Lk={Lk} C={C} H={heads}")
     ws = _workspace(workspace, ws_bytes, dev)
@@ -466,5 +475,6 @@ def cross_apb_forward(a_q: torch.Tensor, a_k: torch.Tensor, s_q, s_k, pair_bias:
         check(L.kfh_cross_apb_forward(aq.data_ptr(), ak.data_ptr(), _ptr(sq), _ptr(sk), pb.data_ptr(),
                                       _io_dtype(pb), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
                                       out.data_ptr(), ws.data_ptr(), ws_bytes, W, Lq, Lk, C, heads,
-                                      cond_channels, float(eps), _io_dtype(aq), _stream(dev)))
+                                      cond_channels, 1 if apply_norm else 0, float(eps), _io_dtype(aq), arith,
+                                      _stream(dev)))
     return out

@@ -39,7 +39,7 @@ def test_size_queries_and_argument_errors_need_no_gpu():
     assert 0 < w1 < w2 and w1 % 256 == 0
     assert lib.kfh_transition_workspace_bytes(1000, 128, 2) == 0       # fused pair kernel
     assert lib.kfh_transition_workspace_bytes(1000, 384, 4) > 0
-    assert lib.kfh_apb_packed_bytes(384, 16, 0) > 0 and lib.kfh_apb_packed_bytes(384, 5, 0) == 0
+    assert lib.kfh_apb_packed_bytes(384, 16, 0, 0) > 0 and lib.kfh_apb_packed_bytes(384, 5, 0, 0) == 0
     # argument checks run before any GPU call
     rc = lib.kfh_trimul_forward(None, None, None, None, None, None, 0, 1, 8, 64, 0, 1e-5, 0, None)
     assert rc == -2 and b"C=64" in lib.kfh_last_error()
@@ -209,10 +209,10 @@ def test_recurrence_window_and_static_entry_points_check_arguments_without_gpu()
     rc = lib.kfh_parcae_step(None, None, None, None, None, 10, 128, 1e-5, 0, None)
     assert rc == -1, lib.kfh_last_error()
     # local attention windows: channels a multiple of 32, head dim at most 64
-    assert lib.kfh_cross_apb_packed_bytes(128, 4, 0) > 0 and lib.kfh_cross_apb_packed_bytes(128, 4, 64) > lib.kfh_cross_apb_packed_bytes(128, 4, 0)
-    assert lib.kfh_cross_apb_packed_bytes(128, 1, 0) == 0 and lib.kfh_cross_apb_packed_bytes(100, 4, 0) == 0
-    w1 = lib.kfh_cross_apb_workspace_bytes(10, 32, 128, 128, 4, 0)
-    w2 = lib.kfh_cross_apb_workspace_bytes(20, 32, 128, 128, 4, 0)
+    assert lib.kfh_cross_apb_packed_bytes(128, 4, 0, 0) > 0 and lib.kfh_cross_apb_packed_bytes(128, 4, 64, 0) > lib.kfh_cross_apb_packed_bytes(128, 4, 0, 0)
+    assert lib.kfh_cross_apb_packed_bytes(128, 1, 0, 0) == 0 and lib.kfh_cross_apb_packed_bytes(100, 4, 0, 0) == 0
+    w1 = lib.kfh_cross_apb_workspace_bytes(10, 32, 128, 128, 4, 0, 0)
+    w2 = lib.kfh_cross_apb_workspace_bytes(20, 32, 128, 128, 4, 0, 0)
     assert 0 < w1 < w2
     # allocation-free transition: 8 MiB of static scratch; a request beyond it is refused before
     # anything touches the GPU, with the limit in the message

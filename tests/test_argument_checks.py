@@ -105,22 +105,32 @@ def test_transition_and_bias_argument_checks(env):
     _expect(lib, lib.kfh_pair_bias_project(p[0], p[1], p[2], 1, 64, 128, 40, 1e-5, 0, None), EUNSUPPORTED, "H=40")
     _expect(lib, lib.kfh_pair_bias_project(None, p[1], p[2], 1, 64, 128, 16, 1e-5, 0, None), EINVAL)
     _expect(lib, lib.kfh_pair_bias_project(p[0], p[1], p[2], 1, 0, 128, 16, 1e-5, 0, None), EINVAL)
-    assert lib.kfh_bias_tiles_bytes(2, 16, 100) == 2 * 16 * 4 * 4 * 2048          # 4 x 4 blocks of 2 KiB
-    _expect(lib, lib.kfh_bias_tiles_from_dense(None, 0, p[0], 1, 16, 100, None), EINVAL)
-    _expect(lib, lib.kfh_bias_tiles_from_dense(p[0], 2, p[1], 1, 16, 100, None), EINVAL, "io_dtype")
+    assert lib.kfh_bias_tiles_bytes(2, 16, 100, 0) == 2 * 16 * 4 * 4 * 2048       # 4 x 4 blocks of 2 KiB
+    assert lib.kfh_bias_tiles_bytes(2, 16, 100, 1) == 2 * 16 * 4 * 4 * 4096       # fp32 tiles
+    assert lib.kfh_bias_tiles_bytes(2, 16, 100, 2) == 0
+    _expect(lib, lib.kfh_bias_tiles_from_dense(None, 0, p[0], 1, 16, 100, 0, None), EINVAL)
+    _expect(lib, lib.kfh_bias_tiles_from_dense(p[0], 2, p[1], 1, 16, 100, 0, None), EINVAL, "io_dtype")
+    _expect(lib, lib.kfh_bias_tiles_from_dense(p[0], 0, p[1], 1, 16, 100, 7, None), EINVAL, "arith")
 
 
 def test_pair_bias_attention_argument_checks(env):
     lib, p, _ = env
-    need = lib.kfh_apb_workspace_bytes(2, 100, 384, 16, 0)
-    assert need > 0 and lib.kfh_apb_workspace_bytes(2, 100, 384, 5, 0) == 0       # head dim 76.8
-    assert lib.kfh_apb_workspace_bytes(2, 100, 384, 2, 0) == 0                    # head dim 192 > 64
+    need = lib.kfh_apb_workspace_bytes(2, 100, 384, 16, 0, 0)
+    assert need > 0 and lib.kfh_apb_workspace_bytes(2, 100, 384, 5, 0, 0) == 0    # head dim 76.8
+    assert lib.kfh_apb_workspace_bytes(2, 100, 384, 2, 0, 0) == 0                 # head dim 192 > 64
+    # fp32 arithmetic: three bf16 parts of everything
+    assert lib.kfh_apb_workspace_bytes(2, 100, 384, 16, 0, 1) > 2 * need
+    assert lib.kfh_apb_workspace_bytes(2, 100, 384, 16, 0, 2) == 0
+    assert lib.kfh_apb_packed_bytes(384, 16, 0, 1) > 2 * lib.kfh_apb_packed_bytes(384, 16, 0, 0)
     f = lib.kfh_apb_forward
 
     def call(a=p[0], s=None, tiles=p[1], mask=p[2], blob=p[3], res=None, out=p[4], ws=p[5], ws_bytes=need,
-             S=2, L=100, C=384, H=16, Cs=0, norm=1, eps=1e-5, io=0):
-        return f(a, s, tiles, mask, blob, res, out, ws, ws_bytes, S, L, C, H, Cs, norm, 0, 0, 0, eps, io, None)
+             S=2, L=100, C=384, H=16, Cs=0, norm=1, eps=1e-5, io=0, arith=0):
+        return f(a, s, tiles, mask, blob, res, out, ws, ws_bytes, S, L, C, H, Cs, norm, 0, 0, 0, eps, io, arith,
+                 None)
 
+    _expect(lib, call(arith=3), EUNSUPPORTED, "arith=3")
+    _expect(lib, call(arith=1), EINVAL, "workspace")          # the bf16 workspace size is too small for fp32
     _expect(lib, call(C=400), EUNSUPPORTED, "C=400")
     _expect(lib, call(H=5), EUNSUPPORTED, "H=5")
     _expect(lib, call(S=0), EINVAL, "S=0")
@@ -131,21 +141,25 @@ def test_pair_bias_attention_argument_checks(env):
     _expect(lib, call(ws_bytes=need - 1), EINVAL, "workspace", str(need))
     g = lib.kfh_apb_pack
     w = p[:8]
-    _expect(lib, g(*w, None, None, None, None, None, None, 0, 384, 7, 0, p[8], None), EUNSUPPORTED, "H=7")
-    _expect(lib, g(*w, None, None, None, None, None, None, 3, 384, 16, 0, p[8], None), EINVAL, "w_dtype")
-    _expect(lib, g(*w[:2], None, *w[3:], None, None, None, None, None, None, 0, 384, 16, 0, p[8], None), EINVAL, "null")
-    _expect(lib, g(*w, None, None, None, None, None, None, 0, 768, 16, 384, p[8], None), EINVAL, "AdaLN")
+    _expect(lib, g(*w, None, None, None, None, None, None, 0, 384, 7, 0, 0, p[8], None), EUNSUPPORTED, "H=7")
+    _expect(lib, g(*w, None, None, None, None, None, None, 3, 384, 16, 0, 0, p[8], None), EINVAL, "w_dtype")
+    _expect(lib, g(*w[:2], None, *w[3:], None, None, None, None, None, None, 0, 384, 16, 0, 0, p[8], None), EINVAL, "null")
+    _expect(lib, g(*w, None, None, None, None, None, None, 0, 768, 16, 384, 0, p[8], None), EINVAL, "AdaLN")
+    _expect(lib, g(*w, None, None, None, None, None, None, 0, 384, 16, 0, 5, p[8], None), EUNSUPPORTED, "arith=5")
 
 
 def test_window_attention_and_recurrence_argument_checks(env):
     lib, p, _ = env
-    need = lib.kfh_cross_apb_workspace_bytes(6, 32, 128, 128, 4, 0)
+    need = lib.kfh_cross_apb_workspace_bytes(6, 32, 128, 128, 4, 0, 0)
+    assert lib.kfh_cross_apb_workspace_bytes(6, 32, 128, 128, 4, 0, 1) > 2 * need
     f = lib.kfh_cross_apb_forward
 
     def call(aq=p[0], ak=p[1], sq=None, sk=None, bias=p[2], bdt=0, mask=p[3], blob=p[4], res=None, out=p[5],
-             ws=p[6], ws_bytes=need, W=6, Lq=32, Lk=128, C=128, H=4, Cs=0, io=0):
-        return f(aq, ak, sq, sk, bias, bdt, mask, blob, res, out, ws, ws_bytes, W, Lq, Lk, C, H, Cs, 1e-5, io, None)
+             ws=p[6], ws_bytes=need, W=6, Lq=32, Lk=128, C=128, H=4, Cs=0, io=0, norm=1, arith=0):
+        return f(aq, ak, sq, sk, bias, bdt, mask, blob, res, out, ws, ws_bytes, W, Lq, Lk, C, H, Cs, norm, 1e-5,
+                 io, arith, None)
 
+    _expect(lib, call(arith=4), EUNSUPPORTED, "arith=4")
     _expect(lib, call(C=100), EUNSUPPORTED, "C=100")
     _expect(lib, call(W=0), EINVAL, "W=0")
     _expect(lib, call(Lk=10000), EUNSUPPORTED, "10000")

@@ -255,8 +255,8 @@ def test_window_attention_flattens_leading_dimensions(rec):
         with pytest.raises(AssertionError):
             cond(a_q, a_k, None, None, bias, mask)
     c0, c1 = rec.of("kfh_cross_apb_forward")
-    assert c0[12:18] == (B * W, Lq, Lk, C, H, 0) and c0[2] is None and c0[3] is None
-    assert c1[12:18] == (B * W, Lq, Lk, C, H, Cs) and c1[2] and c1[3]
+    assert c0[12:19] == (B * W, Lq, Lk, C, H, 0, 1) and c0[2] is None and c0[3] is None
+    assert c1[12:19] == (B * W, Lq, Lk, C, H, Cs, 1) and c1[2] and c1[3]
     assert c0[8] is None, "the module's forward returns the update without a residual"
     assert c0[5] == 0, "bf16 pair bias is passed as it is"
 
@@ -310,10 +310,51 @@ def test_pair_bias_attention_sharing_flags(rec):
     with torch.no_grad():
         layers.hip_attention_pair_bias(plain, x, x, torch.zeros(2, 16, L, L, dtype=torch.bfloat16),
                                        torch.ones(2, L, dtype=torch.bool))
-        with pytest.raises(NotImplementedError):
-            layers.hip_attention_pair_bias(plain, x, x.clone(), torch.zeros(2, 16, L, L), torch.ones(2, L))
+        # different tensors on the two sides: the cross entry, already normalised (apply_norm = 0)
+        xk = torch.zeros(2, 2 * L, 384, dtype=torch.bfloat16)
+        y = layers.hip_attention_pair_bias(plain, x, xk, torch.zeros(2, 16, L, 2 * L, dtype=torch.bfloat16),
+                                           torch.ones(2, 2 * L, dtype=torch.bool))
+        assert y.shape == x.shape
     fn = rec.of("kfh_apb_forward")[-1]
     assert fn[9:15] == (2, L, 384, 16, 0, 0) and fn[15:18] == (1, 1, 0) and fn[1] is None
+    assert fn[20] == 0, "bf16 arithmetic for bf16 activations"
+    cr = rec.of("kfh_cross_apb_forward")[-1]
+    # ..., W, Lq, Lk, C, H, Cs, apply_norm, eps, io_dtype, arith
+    assert cr[12:19] == (2, L, 2 * L, 384, 16, 0, 0) and cr[2] is None and cr[3] is None and cr[21] == 0
+
+
+def test_fp32_arithmetic_is_selected_for_fp32_diffusion_calls(rec, monkeypatch):
+    """The reference runs its diffusion stack in fp32 outside autocast (model/model.py:419): fp32
+    activations at a diffusion call site select KFH_ARITH_F32 (blob, bias tiles, workspace and
+    forward all made for it); the confidence call site, bf16 activations and autocast keep bf16."""
+    from kfold_amd import layers
+
+    L, C, H, Cs, S = 40, 256, 8, 128, 2
+    att = layers.SelfAttentionPairBias(C, H, Cs, "diffusion_global").eval()
+    a32 = torch.zeros(1, S, L, C)
+    s32 = torch.zeros(1, S, L, Cs)
+    bias = torch.zeros(1, 1, H, L, L)
+    mask = torch.ones(1, 1, L, dtype=torch.bool)
+    with torch.no_grad():
+        att(a32, s32, bias, mask)
+        att(a32.bfloat16(), s32.bfloat16(), bias, mask)
+        with monkeypatch.context() as mp:          # autocast("cuda") cannot be entered without a GPU
+            mp.setattr(torch, "is_autocast_enabled", lambda *a: True)
+            att(a32, s32, bias, mask)
+        att.arith = "bf16"
+        att(a32, s32, bias, mask)
+        conf = layers.SelfAttentionPairBias(C, H, None, "confidence").eval()
+        conf(a32, None, bias, mask)
+        win = layers.CrossAttentionPairBias(128, 4, None).eval()
+        win(torch.zeros(3, 32, 128), torch.zeros(3, 128, 128), None, None, torch.zeros(3, 4, 32, 128),
+            torch.ones(3, 128, dtype=torch.bool))
+    fw = rec.of("kfh_apb_forward")
+    assert [c[20] for c in fw] == [1, 0, 0, 0, 0]
+    packs = rec.of("kfh_apb_pack")
+    assert [c[18] for c in packs] == [1, 0, 0], "one blob per arithmetic, re-packed when it changes"
+    tiles = rec.of("kfh_bias_tiles_from_dense")
+    assert [c[6] for c in tiles] == [1, 0, 0, 0, 0]
+    assert rec.of("kfh_cross_apb_forward")[-1][21] == 1 and rec.of("kfh_cross_apb_pack")[-1][24] == 1
 
 
 def test_transition_rows_and_mask_plumbing(rec):

@@ -188,3 +188,109 @@ def test_cross_attention_local_windows(cond):
         want2 = ref(aq2.float(), ak2.float(), f(sq2), f(sk2), b2, m2)
         got2 = hip(aq2.to(DEV), ak2.to(DEV), d(sq2), d(sk2), b2.to(DEV), m2.to(DEV))
     assert_close(got2, want2, "cross attention, 20 x 70 windows", auto_scale=True)
+
+
+# ---------------------------------------------------------------------------------------------
+# fp32 arithmetic of the diffusion stack (reference: model/model.py:419 runs it outside autocast,
+# kernels/triton/attention_pair_bias/dispatch.py:439,453 with fp32_dot_precision="ieee")
+# ---------------------------------------------------------------------------------------------
+F32_MAX_ABS = 1e-4          # against the fp32 oracle; bf16 arithmetic is at ~1e-2 on these inputs
+
+
+@pytest.mark.parametrize("s_shared", [False, True])
+def test_apb_diffusion_variant_fp32_arithmetic(s_shared):
+    """Config 4b shape family with fp32 activations: 5 samples share one pair bias, c_a 768,
+    16 heads x 48, AdaLN conditioning, 12 % of the keys padded — fp32-accurate on the bf16 matrix
+    cores (three-way operand split)."""
+    from kfold_amd.layers import SelfAttentionPairBias
+    from oracle import torch_path as O
+
+    print(f"case apb diffusion fp32 arithmetic s_shared={s_shared}", flush=True)
+    ref, hip = _pair(O.SelfAttentionPairBias, SelfAttentionPairBias, (768, 16, 384, "diffusion_global"),
+                     seed=6, std=0.03, tweak=_affine)
+    L, S = 100, 5
+    g = torch.Generator().manual_seed(8)
+    a = torch.randn(1, S, L, 768, generator=g)
+    s = torch.randn(1, 1 if s_shared else S, L, 384, generator=g)
+    bias = torch.randn(1, 1, 16, L, L, generator=g)
+    mask = torch.ones(1, 1, L, dtype=torch.bool)
+    mask[..., L - 12:] = False
+    with torch.no_grad():
+        want = ref(a, s.expand(1, S, L, 384), bias, mask)
+        got = hip(a.to(DEV), s.to(DEV), bias.to(DEV), mask.to(DEV))
+        assert got.shape == a.shape and got.dtype == torch.float32
+        e = assert_close(got, want, "apb diffusion variant, fp32 arithmetic", max_abs=F32_MAX_ABS, mean_abs=1e-5,
+                         rel_fro=1e-5)
+        print(e, flush=True)
+        hip.arith = "bf16"                             # the same call in bf16 arithmetic, for scale
+        got16 = hip(a.to(DEV), s.to(DEV), bias.to(DEV), mask.to(DEV))
+    e16 = assert_close(got16, want, "apb diffusion variant, bf16 arithmetic on fp32 tensors", auto_scale=True)
+    assert e["max_abs"] < 0.02 * e16["max_abs"], (e, e16)
+
+
+@pytest.mark.parametrize("cond", [False, True])
+def test_cross_attention_local_windows_fp32_arithmetic(cond):
+    """32 x 128 windows (and an odd 20 x 70 shape) in fp32 arithmetic, a fully masked window and a
+    partially masked one included."""
+    from kfold_amd.layers import CrossAttentionPairBias
+    from oracle import torch_path as O
+
+    print(f"case cross attention windows fp32 arithmetic cond={cond}", flush=True)
+    cs = 128 if cond else None
+    ref, hip = _pair(O.CrossAttentionPairBias, CrossAttentionPairBias, (128, 4, cs), seed=12, std=0.05,
+                     tweak=_affine)
+    S, W, Lq, Lk = 2, 11, 32, 128
+    g = torch.Generator().manual_seed(14)
+    aq = torch.randn(S, W, Lq, 128, generator=g)
+    ak = torch.randn(S, W, Lk, 128, generator=g)
+    sq = torch.randn(S, W, Lq, 128, generator=g) if cond else None
+    sk = torch.randn(S, W, Lk, 128, generator=g) if cond else None
+    bias = torch.randn(1, W, 4, Lq, Lk, generator=g)
+    mask = torch.rand(1, W, Lk, generator=g) > 0.2
+    mask[0, 3] = False
+    mask[0, 7, 40:] = False
+    d = lambda t: None if t is None else t.to(DEV)
+    with torch.no_grad():
+        want = ref(aq, ak, sq, sk, bias, mask)
+        got = hip(aq.to(DEV), ak.to(DEV), d(sq), d(sk), bias.to(DEV), mask.to(DEV))
+    assert got.dtype == torch.float32
+    print(assert_close(got, want, "cross attention windows, fp32 arithmetic", max_abs=F32_MAX_ABS, mean_abs=1e-5,
+                       rel_fro=1e-5), flush=True)
+    Lq2, Lk2 = 20, 70
+    c = lambda t, n: None if t is None else t[:1, :, :n].contiguous()
+    b2, m2 = bias[:, :, :, :Lq2, :Lk2].contiguous(), mask[:, :, :Lk2].contiguous()
+    with torch.no_grad():
+        want2 = ref(c(aq, Lq2), c(ak, Lk2), c(sq, Lq2), c(sk, Lk2), b2, m2)
+        got2 = hip(d(c(aq, Lq2)), d(c(ak, Lk2)), d(c(sq, Lq2)), d(c(sk, Lk2)), b2.to(DEV), m2.to(DEV))
+    assert_close(got2, want2, "cross attention, 20 x 70 windows, fp32 arithmetic", max_abs=F32_MAX_ABS,
+                 mean_abs=1e-5, rel_fro=1e-5)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_functional_entry_with_different_query_and_key_tensors(dtype):
+    """``attention_pair_bias(module, x_q, x_k, ...)`` as CrossAttentionPairBias.forward calls it
+    (layers/folding/attention_pair_bias.py:250-258): both sides already normalised, Lq != Lk."""
+    from kfold_amd.layers import CrossAttentionPairBias, hip_attention_pair_bias
+    from oracle import torch_path as O
+
+    print(f"case functional entry, x_q != x_k, {dtype}", flush=True)
+    ref, hip = _pair(O.CrossAttentionPairBias, CrossAttentionPairBias, (128, 4, None), seed=15, std=0.05)
+    with torch.no_grad():
+        ref.linear_q.bias.copy_(0.2 * torch.randn(128, generator=torch.Generator().manual_seed(9)))
+    hip.load_state_dict(ref.state_dict())
+    W, Lq, Lk = 9, 32, 128
+    g = torch.Generator().manual_seed(16)
+    xq = torch.randn(2, W, Lq, 128, generator=g).to(dtype)
+    xk = torch.randn(2, W, Lk, 128, generator=g).to(dtype)
+    bias = torch.randn(1, W, 4, Lq, Lk, generator=g)
+    mask = torch.rand(1, W, Lk, generator=g) > 0.3
+    with torch.no_grad():
+        want = O.torch_attention_pair_bias(ref, xq.float(), xk.float(), bias, mask)
+        got = hip_attention_pair_bias(hip, xq.to(DEV), xk.to(DEV), bias.to(DEV), mask.to(DEV),
+                                      call_site="diffusion_local")
+    assert got.shape == xq.shape and got.dtype == dtype
+    if dtype == torch.float32:
+        assert_close(got, want, "functional cross entry, fp32 arithmetic", max_abs=F32_MAX_ABS, mean_abs=1e-5,
+                     rel_fro=1e-5)
+    else:
+        assert_close(got, want, "functional cross entry, bf16", auto_scale=True)
