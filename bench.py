@@ -63,24 +63,37 @@ def kernel_sources_digest() -> str:
 
 def read_traffic_profile(n: int) -> tuple[dict, str | None]:
     """{kernel name: (read MB, write MB)} from the committed counter summary, and the reason it
-    cannot be used (None when it can): other N, missing, or taken from other kernel sources."""
+    cannot be used (None when it can): other N, missing, or measured on other machine code.  A row
+    is used only while the kernel in the library being run has the instruction-stream digest the
+    summary lists for it (``kfold_amd/kernel_isa.json``, written by the build)."""
     if n != 768:
         return {}, f"the committed counter runs are at N=768, not N={n}"
     try:
         text = open(TRAFFIC_PROFILE).read()
     except OSError:
         return {}, "no counter summary under profiles/"
-    m = re.search(r"kernel sources digest: `([0-9a-f]+)`", text)
-    if not m or m.group(1) != kernel_sources_digest():
-        return {}, "the counter summary under profiles/ was taken from other kernel sources"
+    try:
+        from kfold_amd.build import ISA_JSON
+
+        built = json.loads(ISA_JSON.read_text())
+    except (OSError, ValueError):
+        return {}, "kfold_amd/kernel_isa.json is missing: the library was not built by kfold_amd.build"
+    measured = {}            # table name -> digest the summary was measured on
+    for line in text.splitlines():
+        cells = [c.strip() for c in line.split("|")]
+        if len(cells) >= 5 and cells[1].startswith("kfh::") and cells[2].startswith("`_Z"):
+            if built.get(cells[2].strip("`")) == cells[3].strip("`"):
+                measured[cells[1]] = cells[3]
     rows = {}
     for line in text.splitlines():
         cells = [c.strip() for c in line.split("|")]
-        if len(cells) >= 8 and cells[1].startswith("kfh::"):
+        if len(cells) >= 8 and cells[1] in measured:
             try:
                 rows[cells[1]] = (float(cells[5]), float(cells[6]))
             except ValueError:
                 pass
+    if not rows:
+        return {}, "the counter summary under profiles/ was taken on other machine code of every kernel"
     return rows, None
 
 
@@ -374,6 +387,81 @@ def config_table() -> list[dict]:
         ms = statistics.median(event_time_ms(lambda: m(ad, scd, bd, md), 10))
         rows.append(dict(config="C4b", what="APB diffusion N=768 S=5, dense bias in", hip_ms=ms,
                          tflops=3.85e10 / ms / 1e9, roof=f"MFMA {3.85e10 / ms / 1e9 / PEAK_BF16_TFLOPS * 100:.1f} %"))
+        rows += shipping_dim_rows(dev, lambda fn: statistics.median(event_time_ms(fn, 10)))
+    return rows
+
+
+def shipping_dim_rows(dev, time_ms, n_wide: int = 768, n_templates: int = 384, n_atoms_windows: int = 24,
+                      n_tokens: int = 768) -> list[dict]:
+    """The widths the shipping model runs at (configs/kfold.yaml of the reference): triangle
+    multiplication and the trunk's TriangularBlock at c_z = 256, triangle attention at c = 64 with
+    4 heads of 16 over a batch of 4 templates, and the diffusion attention in fp32 arithmetic.
+    ``time_ms(fn)`` returns the time of one call of ``fn`` in ms."""
+    import torch
+
+    from kfold_amd import layers, modules, primitives, synthetic
+
+    rows = []
+    n = n_wide
+    tok = synthetic.token_mask(n, synthetic.n_pad_for(n, 0.12))
+    pm = synthetic.pair_mask_from_tokens(tok).to(dev)
+    g = torch.Generator().manual_seed(3)
+    zd = torch.randn(1, n, n, 256, generator=g).bfloat16().to(dev)
+    fl_tm = 2 * n**3 * 256 + n * n * (8 * 256 * 256 + 2 * 256 * 256 + 2 * 256 * 256)      # 2 N^3 D + N^2 (8 C D + 2 D C + 2 C^2) with C = D = 256
+    for what, mk in (("tri-mul out C=256", lambda: primitives.TriangleMultiplicationOutgoing(256)),
+                     ("tri-mul in C=256", lambda: primitives.TriangleMultiplicationIncoming(256))):
+        m = mk().eval()
+        synthetic.init_weights_(m, 0)
+        m.to(dev)
+        ms = time_ms(lambda: m(zd, pm))
+        rows.append(dict(config="F2", what=f"{what} N={n}", hip_ms=ms, tflops=fl_tm / ms / 1e9,
+                         roof=f"MFMA {fl_tm / ms / 1e9 / PEAK_BF16_TFLOPS * 100:.1f} %"))
+    blk = modules.TriangularBlock(256).eval()
+    synthetic.init_weights_(blk, 1)
+    blk.to(dev)
+    fl_blk = 2 * fl_tm + 6 * 256 * 256 * 4 * n * n
+    zin = zd.clone()
+    ms = time_ms(lambda: blk(zin, pm))
+    rows.append(dict(config="F2", what=f"TriangularBlock C=256 N={n} (tri-mul out, in, transition x4)", hip_ms=ms,
+                     tflops=fl_blk / ms / 1e9, roof=f"MFMA {fl_blk / ms / 1e9 / PEAK_BF16_TFLOPS * 100:.1f} %"))
+    del zd, zin
+    n, batch = n_templates, 4
+    xd = torch.randn(batch, n, n, 64, generator=g).bfloat16().to(dev)
+    pmt = synthetic.pair_mask_from_tokens(synthetic.token_mask(n, synthetic.n_pad_for(n, 0.1))).expand(batch, n, n)
+    pmt = pmt.contiguous().to(dev)
+    fl_ta = batch * (4 * n**3 * 64 + n * n * (8 * 64 * 64 + 2 * 64 * 4 + 2 * 64 * 64))
+    for what, mk in (("tri-attn start", lambda: primitives.TriangleAttentionStartingNode(64, 4)),
+                     ("tri-attn end", lambda: primitives.TriangleAttentionEndingNode(64, 4))):
+        m = mk().eval()
+        synthetic.init_weights_(m, 2)
+        m.to(dev)
+        ms = time_ms(lambda: m(xd, pmt))
+        rows.append(dict(config="F2", what=f"{what} C=64 4x16, {batch} templates, N={n}", hip_ms=ms,
+                         tflops=fl_ta / ms / 1e9, roof=f"MFMA {fl_ta / ms / 1e9 / PEAK_BF16_TFLOPS * 100:.1f} %"))
+    # diffusion attention on fp32 tensors: fp32 arithmetic (six bf16 part products per k-step)
+    n = n_tokens
+    m = layers.SelfAttentionPairBias(768, 16, 384, "diffusion_global").eval()
+    synthetic.init_weights_(m, 8)
+    m.to(dev)
+    ad = torch.randn(1, 5, n, 768, generator=g).to(dev)
+    scd = torch.randn(1, 5, n, 384, generator=g).to(dev)
+    bd = torch.randn(1, 1, 16, n, n, generator=g).to(dev)
+    md = synthetic.token_mask(n, synthetic.n_pad_for(n, 0.12)).reshape(1, 1, n).to(dev)
+    ms = time_ms(lambda: m(ad, scd, bd, md))
+    fl = 3.85e10 * (n / 768) ** 2
+    rows.append(dict(config="F3", what=f"APB diffusion N={n} S=5, fp32 arithmetic", hip_ms=ms, tflops=fl / ms / 1e9,
+                     roof=f"MFMA {6 * fl / ms / 1e9 / PEAK_BF16_TFLOPS * 100:.1f} % of bf16 peak on the 6x executed products"))
+    W = n_atoms_windows
+    cross = layers.CrossAttentionPairBias(128, 4, 128).eval()
+    synthetic.init_weights_(cross, 9)
+    cross.to(dev)
+    aq, ak = torch.randn(5, W, 32, 128, generator=g).to(dev), torch.randn(5, W, 128, 128, generator=g).to(dev)
+    sq, sk = torch.randn(5, W, 32, 128, generator=g).to(dev), torch.randn(5, W, 128, 128, generator=g).to(dev)
+    cb = torch.randn(1, W, 4, 32, 128, generator=g).to(dev)
+    cm = torch.ones(1, W, 128, dtype=torch.bool).to(dev)
+    ms = time_ms(lambda: cross(aq, ak, sq, sk, cb, cm))
+    rows.append(dict(config="F3", what=f"cross attention, 5 x {W} windows of 32 x 128, fp32 arithmetic", hip_ms=ms,
+                     tflops=None, roof="launch-latency bound"))
     return rows
 
 
@@ -557,7 +645,9 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": f"pairformer_block_N{n}", "n_tokens": n, "n_padded_tokens": h.n_pad,
                    "c_z": 128, "c_s": 384, "tri_heads": "4x32", "apb_heads": "16x24",
-                   "pair_transition_expansion": 2, "single_transition_expansion": 4},
+                   "pair_transition_expansion": 2, "single_transition_expansion": 4,
+                   "schedule": "chain of `steps` blocks; single track of step k on a second stream beside the "
+                               "pair track of step k+1 (serial_schedule_ms_per_step: everything on one stream)"},
         "schedule": "single track of step k on a second stream beside the pair track of step k+1",
         "serial_schedule_ms_per_step": round(timings["serial"], 4),
         "block_tflops": round(fl["block"] / ms_per_step / 1e9, 1),

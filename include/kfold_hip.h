@@ -93,8 +93,12 @@ int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, con
                        int direction, float eps, int io_dtype, void* stream);
 
 /* Same as kfh_trimul_forward but runs only the kernels selected by `stages` (an OR of
- * KFH_STAGE_*); later stages read what earlier ones left in `workspace`.  For profiling and
- * benchmarks of the individual kernels; no counterpart in the reference. */
+ * KFH_STAGE_*).  Later stages read what earlier ones left in `workspace` AND, for
+ * KFH_STAGE_OUT, `z` again (the output gate sigmoid(W_go LN_in(z)) is recomputed from it):
+ * every stage of one op must be given the same, unmodified z (a split around a write to z,
+ * e.g. IN|CORE, then other work, then OUT with out == z, is the intended use — OUT reads a row
+ * of z before it writes it).  For profiling, benchmarks of the individual kernels and callers
+ * that order the write to `out` against other streams; no counterpart in the reference. */
 int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* blob,
                               const void* residual, void* out, void* workspace,
                               size_t workspace_bytes, int B, int N, int C, int direction, float eps,
@@ -127,7 +131,9 @@ int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, co
                         void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                         int H, int ending, float eps, int io_dtype, void* stream);
 
-/* Stage-selective variant, see kfh_trimul_forward_stages. */
+/* Stage-selective variant, see kfh_trimul_forward_stages: KFH_STAGE_OUT of the C = 128, 4-head
+ * path reads `x` again for the gate sigmoid(W_g LN(x)) (other widths keep their gate in the
+ * workspace); give every stage the same, unmodified x. */
 int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* blob,
                                const void* residual, void* out, void* workspace,
                                size_t workspace_bytes, int B, int N, int C, int H, int ending,
@@ -164,7 +170,12 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
  * fail with KFH_EINVAL (e.g. C = 384, expansion 4: up to 2184 rows).  All calls on one GPU
  * share the array: calls that may overlap in time on one GPU (different streams or threads)
  * race; calls on one stream are ordered.  Results are bit-identical to
- * kfh_transition_forward. */
+ * kfh_transition_forward.
+ * Set-up: kfh_transition_static_scratch_bytes() also resolves and keeps the array's address on
+ * the CURRENT device; call it once per device (with that device current) before the first
+ * kfh_transition_forward_static there if that first call must do no lookup (graph capture).
+ * kfh_transition_forward_static uses the array of the current device: `stream` must belong to
+ * the device that is current at the call. */
 size_t kfh_transition_static_scratch_bytes(void);
 int kfh_transition_forward_static(const void* x, const void* blob, const void* residual,
                                   const uint8_t* mask, void* out, long long rows, int C, int expansion,

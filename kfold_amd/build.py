@@ -44,6 +44,51 @@ def _compile(src: Path, obj: Path, verbose: bool) -> None:
         print(err, file=sys.stderr)
 
 
+# kernel files whose machine code the committed profiles were measured on
+ISA_FILES = ("trimul", "contract", "triattn", "flash", "transition", "pairbias")
+ISA_JSON = ROOT / "kernel_isa.json"
+
+
+def _isa_of(src: Path) -> dict[str, str]:
+    """{mangled kernel name: digest of its gfx950 instruction stream} for one source file.  Labels,
+    directives and comments are dropped, so the digest changes only when an instruction does."""
+    import hashlib
+    import re
+
+    res = subprocess.run([HIPCC, *FLAGS, "--cuda-device-only", "-S", str(src), "-o", "-"],
+                         capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc -S failed for {src.name}:\n{res.stderr[-2000:]}")
+    out: dict[str, list[str]] = {}
+    cur = None
+    for line in res.stdout.splitlines():
+        m = re.match(r"^(_Z\w+):", line)
+        if m:
+            cur = m.group(1)
+            out[cur] = []
+            continue
+        if cur is None:
+            continue
+        code = line.split(";")[0].strip()
+        if code.startswith(".Lfunc_end"):
+            cur = None
+        elif code and not code.startswith("."):
+            out[cur].append(code)
+    return {k: hashlib.sha256("\n".join(v).encode()).hexdigest()[:16] for k, v in out.items()}
+
+
+def isa_digests(jobs: int = 8) -> dict[str, str]:
+    """Digest of the compiled instruction stream of every kernel of the hot-path files: what a
+    measurement (a rocprofv3 summary under profiles/) is valid for.  Edits that leave a kernel's
+    machine code unchanged (comments, new helpers, other kernels) keep its digest."""
+    srcs = [CSRC / f"{name}.hip" for name in ISA_FILES]
+    merged: dict[str, str] = {}
+    with ThreadPoolExecutor(max_workers=jobs) as ex:
+        for d in ex.map(_isa_of, srcs):
+            merged.update(d)
+    return dict(sorted(merged.items()))
+
+
 def build(verbose: bool = False, jobs: int | None = None) -> Path:
     objdir = CSRC / "_obj"
     objdir.mkdir(exist_ok=True)
@@ -58,6 +103,9 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
     res = subprocess.run(cmd, capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"link failed:\n{res.stderr}")
+    import json
+
+    ISA_JSON.write_text(json.dumps(isa_digests(), indent=1) + "\n")
     return LIB
 
 

@@ -465,7 +465,15 @@ int kfh_transition_forward(const void* x, const void* blob, const void* residual
                                    expansion, eps, io_dtype, stream);
 }
 
-size_t kfh_transition_static_scratch_bytes(void) { return kStaticScratchBytes; }
+// Also the set-up call: it looks up (and keeps) the scratch array's address on the current device, so
+// that a later kfh_transition_forward_static on this device does no symbol lookup — callers that
+// capture a graph or run a tight loop call this once per device beforehand.  The size is returned
+// whether or not a device is present.
+size_t kfh_transition_static_scratch_bytes(void) {
+    void* p = nullptr;
+    (void)static_scratch_ptr(&p);
+    return kStaticScratchBytes;
+}
 
 int kfh_transition_forward_static(const void* x, const void* blob, const void* residual,
                                   const uint8_t* mask, void* out, long long rows, int C, int expansion,
