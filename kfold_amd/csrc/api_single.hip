@@ -338,7 +338,7 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
 // transition for any channel count (token track); C = 128 uses the fused pair kernel
 // ------------------------------------------------------------------------------------------
 size_t kfh_transition_packed_bytes(int C, int expansion) {
-    if (C == kC && (expansion == 2 || expansion == 4)) return align_up(transition_blob_bytes(expansion));
+    if (transition_fused(C, expansion)) return align_up(transition_blob_bytes(expansion, C));
     if (C <= 0 || C % 128 || C > 2048 || expansion < 1 || expansion > 8) return 0;
     return GtLayout(C, expansion).total;
 }
@@ -353,20 +353,21 @@ int kfh_transition_pack(const void* ln_w, const void* ln_b, const void* swiglu_w
     char* b = static_cast<char*>(blob);
     const int hid = C * expansion;
     const size_t wsz = w_dtype == KFH_F32 ? 4 : 2;
-    if (C == kC && (expansion == 2 || expansion == 4)) {
+    if (transition_fused(C, expansion)) {
         const int nstep = hid / 32;
+        const size_t blk = (size_t)32 * C * 2;          // one 32-row block of C channels
         for (int s = 0; s < nstep; ++s) {
-            char* step = b + (size_t)s * 3 * kBlockBytes;
+            char* step = b + (size_t)s * 3 * blk;
             // u rows are packed times -log2(e) and W_out times -ln(2): the kernel then needs
             // u' v / (1 + exp2(u')) with u' = -log2(e) u, one multiply less per element
             launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, 32 * s, 1, ROW_NATURAL, K_NATURAL, -kLog2e, step, stream);
             launch_pack_blocks(swiglu_w, w_dtype, 32, C, C, hid + 32 * s, 1, ROW_NATURAL, K_NATURAL, 1.f,
-                               step + kBlockBytes, stream);
+                               step + blk, stream);
             // W_out[:, 32s .. 32s+31]: a 32-wide column slice of the [C, hid] matrix
             launch_pack_blocks(static_cast<const char*>(out_w) + (size_t)32 * s * wsz, w_dtype, C, 32, hid,
-                               0, 4, ROW_INTERLEAVE4, K_ACC, -1.0f / kLog2e, step + 2 * kBlockBytes, stream);
+                               0, C / 32, ROW_INTERLEAVE4, K_ACC, -1.0f / kLog2e, step + 2 * blk, stream);
         }
-        float* ln = reinterpret_cast<float*>(b + (size_t)nstep * 3 * kBlockBytes);
+        float* ln = reinterpret_cast<float*>(b + (size_t)nstep * 3 * blk);
         launch_copy_f32(ln_w, w_dtype, ln, C, 1.f, stream);
         launch_copy_f32(ln_b, w_dtype, ln + C, C, 0.f, stream);
     } else {
@@ -382,7 +383,7 @@ int kfh_transition_pack(const void* ln_w, const void* ln_b, const void* swiglu_w
 }
 
 size_t kfh_transition_workspace_bytes(long long rows, int C, int expansion) {
-    if (C == kC && (expansion == 2 || expansion == 4)) return 0;
+    if (transition_fused(C, expansion)) return 0;
     if (rows <= 0 || kfh_transition_packed_bytes(C, expansion) == 0) return 0;
     return align_up((size_t)rows * C * 2) + align_up((size_t)rows * C * expansion * 2);
 }
@@ -401,12 +402,13 @@ int transition_forward_impl(const void* x, const void* blob, const void* residua
     if (rows == 0) return KFH_OK;
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     const char* b = static_cast<const char*>(blob);
-    if (C == kC && (expansion == 2 || expansion == 4)) {
-        KFH_TRY(launch_pair_transition(x, io_dtype, b, expansion, residual, mask, out, rows, eps, stream),
+    if (transition_fused(C, expansion)) {
+        KFH_TRY(C == kC ? launch_pair_transition(x, io_dtype, b, expansion, residual, mask, out, rows, eps, stream)
+                        : launch_pair_transition_wide(x, io_dtype, b, expansion, residual, mask, out, rows, eps, stream, C),
                 "pair transition");
         return check_launch("transition_forward");
     }
-    if (mask) return fail(KFH_EUNSUPPORTED, "transition_forward: the row mask is built for C=128 only");
+    if (mask) return fail(KFH_EUNSUPPORTED, "transition_forward: the row mask is built for C=128 and C=256 only");
     if (rows > 0x7fffffffLL) return fail(KFH_EUNSUPPORTED, "transition_forward: too many rows");
     const size_t need = kfh_transition_workspace_bytes(rows, C, expansion);
     if (!workspace || workspace_bytes < need)

@@ -106,13 +106,20 @@ int triattn_generic_forward(const void* x, int io_dtype, const uint8_t* mask, co
                             int stages, hipStream_t stream);
 
 // ---- pair transition (transition.hip) ----------------------------------------------------
-// Packed blob (C = 128, expansion E): 4E steps x 24 KiB { u block, v block, W_out slice of the
-// step's 32 hidden channels as 4 blocks x 2 k-steps (ROW_INTERLEAVE4, K_ACC) }, then fp32 LN
-// gamma, beta.
-inline size_t transition_blob_bytes(int E) { return (size_t)4 * E * 3 * kBlockBytes + 2 * kC * sizeof(float); }
+// Packed blob (C = 128 or 256, expansion E): C*E/32 steps x { u block, v block, W_out slice of the
+// step's 32 hidden channels as C/32 blocks x 2 k-steps (ROW_INTERLEAVE4, K_ACC) } (24 KiB per step
+// at C = 128, 48 KiB at C = 256), then fp32 LN gamma, beta.
+inline size_t transition_blob_bytes(int E, int C = kC) {
+    return (size_t)(C * E / 32) * 3 * 32 * C * 2 + 2 * (size_t)C * sizeof(float);
+}
+inline bool transition_fused(int C, int E) { return (C == kC || C == 256) && (E == 2 || E == 4); }
 int launch_pair_transition(const void* x, int io_dtype, const char* blob, int expansion,
                            const void* residual, const uint8_t* mask, void* out, long long M,
                            float eps, hipStream_t stream);
+// the same kernel at C = 256 (transition_wide.hip)
+int launch_pair_transition_wide(const void* x, int io_dtype, const char* blob, int expansion,
+                                const void* residual, const uint8_t* mask, void* out, long long M,
+                                float eps, hipStream_t stream, int C);
 
 // ---- pair bias projection (pairbias.hip): blob = one packed block (heads as rows, scaled by
 // log2 e) followed by fp32 LN gamma, beta

@@ -33,7 +33,7 @@ def _affine(ref):
 
 
 @pytest.mark.parametrize("channel,expansion,rows", [(128, 2, 1000), (128, 4, 333), (384, 4, 70),
-                                                     (768, 2, 33)])
+                                                     (768, 2, 33), (256, 4, 1000), (256, 2, 77)])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
 def test_transition_parity(channel, expansion, rows, dtype):
     from kfold_amd.layers import Transition, hip_transition
@@ -50,7 +50,7 @@ def test_transition_parity(channel, expansion, rows, dtype):
         # fused residual (in place) and, for the pair kernel, the row mask
         xin = x.to(DEV).clone()
         mask = (torch.rand(rows, generator=torch.Generator().manual_seed(1)) > 0.3)
-        if channel == 128:
+        if channel in (128, 256):          # the fused pair-track kernels take the row mask
             hip_transition(hip, xin, residual=xin, mask=mask.to(DEV), out=xin)
             want2 = (x.float() + want) * mask[:, None]
             assert (xin.cpu()[~mask] == 0).all()
