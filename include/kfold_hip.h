@@ -145,8 +145,8 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
  * reference runs unfused on every backend.  C = 128 and C = 256 with expansion 2 or 4 (the
  * pair track of the Pairformer block and of the trunk's TriangularBlock,
  * model/modules/tri_stack.py:119-125) run as one fused kernel and need no workspace; other
- * channel counts (multiples of 128 up to 2048: the token track) run as LayerNorm + two MFMA
- * linears through the workspace.
+ * channel counts (multiples of 32 up to 2048: the token track, the C = 64 template stack) run
+ * as LayerNorm + two MFMA linears through the workspace.
  * ------------------------------------------------------------------------------------- */
 size_t kfh_transition_packed_bytes(int C, int expansion);
 
@@ -158,7 +158,7 @@ size_t kfh_transition_workspace_bytes(long long rows, int C, int expansion);
 
 /* out[r,:] = ((residual ? residual[r,:] : 0) + Transition(x[r,:])) * (mask ? mask[r] != 0 : 1)
  * for r < rows; x, out, residual: [rows, C].  `out` may alias `x` and `residual`.  `mask`
- * (C = 128 / 256 only, else NULL) is the final `z * pair_mask` of modules/apo_module.py:172. */
+ * (one byte per row, or NULL) is the final `z * pair_mask` of modules/apo_module.py:172. */
 int kfh_transition_forward(const void* x, const void* blob, const void* residual, const uint8_t* mask,
                            void* out, void* workspace, size_t workspace_bytes, long long rows, int C,
                            int expansion, float eps, int io_dtype, void* stream);

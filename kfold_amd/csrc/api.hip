@@ -22,10 +22,13 @@ const char* kfh_last_error(void) { return kfh::g_err; }
 // ------------------------------------------------------------------------------------------
 namespace {
 bool trimul_wide(int C) { return C == 256; }
+// any other multiple of 32 up to 256 runs on the path assembled from the token-track kernels
+bool trimul_generic(int C) { return C != kC && !trimul_wide(C) && trimul_generic_blob_bytes(C) != 0; }
 }  // namespace
 
 size_t kfh_trimul_packed_bytes(int C) {
     if (trimul_wide(C)) return align_up(trimul_wide_blob_bytes(C));
+    if (trimul_generic(C)) return trimul_generic_blob_bytes(C);
     return C == kC ? align_up(kTmBlobBytes) : 0;
 }
 
@@ -33,13 +36,19 @@ int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w
                     const void* g_in_w, const void* ln_out_w, const void* ln_out_b,
                     const void* p_out_w, const void* g_out_w, int w_dtype, int C, void* blob,
                     void* stream_) {
-    if (C != kC && !trimul_wide(C))
-        return fail(KFH_EUNSUPPORTED, "trimul_pack: C=%d, built for C=128 and C=256", C);
+    if (C != kC && !trimul_wide(C) && !trimul_generic(C))
+        return fail(KFH_EUNSUPPORTED, "trimul_pack: C=%d (a multiple of 32 up to 256)", C);
     if (!dtype_ok(w_dtype)) return fail(KFH_EINVAL, "trimul_pack: bad w_dtype %d", w_dtype);
     if (!p_in_w || !g_in_w || !p_out_w || !g_out_w || !blob)
         return fail(KFH_EINVAL, "trimul_pack: null weight or blob pointer");
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     char* b = static_cast<char*>(blob);
+    if (trimul_generic(C)) {
+        if (trimul_generic_pack(ln_in_w, ln_in_b, p_in_w, g_in_w, ln_out_w, ln_out_b, p_out_w, g_out_w, w_dtype, C,
+                                blob, stream))
+            return fail(KFH_EUNSUPPORTED, "trimul_pack: C=%d not built", C);
+        return check_launch("trimul_pack");
+    }
     if (trimul_wide(C)) {
         size_t o_gate, o_ab, o_out, o_ln, blk;
         trimul_wide_offsets(C, &o_gate, &o_ab, &o_out, &o_ln, &blk);
@@ -79,6 +88,7 @@ int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w
 }
 
 size_t kfh_trimul_workspace_bytes(int N, int C) {
+    if (trimul_generic(C)) return trimul_generic_ws_bytes(N, C);
     if ((C != kC && !trimul_wide(C)) || N <= 0) return 0;
     const size_t np = trimul_np(N);
     const size_t planes_ab = align_up(2 * (size_t)C * np * np * 2);
@@ -97,8 +107,8 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
                               const void* residual, void* out, void* workspace,
                               size_t workspace_bytes, int B, int N, int C, int direction, float eps,
                               int io_dtype, int stages, void* stream_) {
-    if (C != kC && !trimul_wide(C))
-        return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d, built for C=128 and C=256", C);
+    if (C != kC && !trimul_wide(C) && !trimul_generic(C))
+        return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d (a multiple of 32 up to 256)", C);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "trimul_forward: bad shape B=%d N=%d", B, N);
     if (!dtype_ok(io_dtype)) return fail(KFH_EINVAL, "trimul_forward: bad io_dtype %d", io_dtype);
     if (direction != KFH_OUTGOING && direction != KFH_INCOMING)
@@ -114,6 +124,17 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
     const int np = trimul_np(N);
     const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
     char* ws = static_cast<char*>(workspace);
+    if (trimul_generic(C)) {
+        for (int b = 0; b < B; ++b) {       // batch elements (templates) in turn through one workspace
+            const size_t off = (size_t)b * N * N * C * esz;
+            const int rc = trimul_generic_forward(
+                static_cast<const char*>(z) + off, io_dtype, mask + (size_t)b * N * N, static_cast<const char*>(blob),
+                ws, residual ? static_cast<const char*>(residual) + off : nullptr, static_cast<char*>(out) + off, N, C,
+                direction == KFH_INCOMING, eps, stages, stream);
+            if (rc) return fail(KFH_EUNSUPPORTED, "trimul_forward: shape not built (%d)", rc);
+        }
+        return check_launch("trimul_forward");
+    }
     uint16_t* planes_ab = reinterpret_cast<uint16_t*>(ws);
     uint16_t* planes_y = reinterpret_cast<uint16_t*>(ws + align_up(2 * (size_t)C * np * np * 2));
     const char* bl = static_cast<const char*>(blob);

@@ -339,7 +339,7 @@ int kfh_apb_forward(const void* a, const void* s_cond, const void* bias_tiles, c
 // ------------------------------------------------------------------------------------------
 size_t kfh_transition_packed_bytes(int C, int expansion) {
     if (transition_fused(C, expansion)) return align_up(transition_blob_bytes(expansion, C));
-    if (C <= 0 || C % 128 || C > 2048 || expansion < 1 || expansion > 8) return 0;
+    if (C <= 0 || C % 32 || C > 2048 || expansion < 1 || expansion > 8) return 0;
     return GtLayout(C, expansion).total;
 }
 
@@ -408,7 +408,6 @@ int transition_forward_impl(const void* x, const void* blob, const void* residua
                 "pair transition");
         return check_launch("transition_forward");
     }
-    if (mask) return fail(KFH_EUNSUPPORTED, "transition_forward: the row mask is built for C=128 and C=256 only");
     if (rows > 0x7fffffffLL) return fail(KFH_EUNSUPPORTED, "transition_forward: too many rows");
     const size_t need = kfh_transition_workspace_bytes(rows, C, expansion);
     if (!workspace || workspace_bytes < need)
@@ -425,6 +424,7 @@ int transition_forward_impl(const void* x, const void* blob, const void* residua
     LinearArgs q = plain(hid, l.hid, rows, l.hid, b + l.wo, C);
     q.epi = EPI_RESID;
     if (residual) { q.aux = residual; q.aux_dtype = io_dtype; q.ld_aux = C; }
+    q.mask = mask;
     q.out = out; q.out_dtype = io_dtype; q.ldo = C;
     KFH_TRY(launch_linear(q, stream), "linear");
     return check_launch("transition_forward");

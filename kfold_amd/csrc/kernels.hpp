@@ -43,6 +43,16 @@ void launch_trimul_out(const uint16_t* planes_y, const void* z, const char* blob
                        const void* residual, void* out, int io_dtype, int N, int Np, float eps,
                        hipStream_t stream);
 
+// any other width that is a multiple of 32 (trimul_generic.hip), from the token-track kernels
+size_t trimul_generic_blob_bytes(int C);
+size_t trimul_generic_ws_bytes(int N, int C);
+int trimul_generic_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w, const void* g_in_w,
+                        const void* ln_out_w, const void* ln_out_b, const void* p_out_w, const void* g_out_w,
+                        int w_dtype, int C, void* blob, hipStream_t stream);
+int trimul_generic_forward(const void* z, int io_dtype, const uint8_t* mask, const char* blob, char* ws,
+                           const void* residual, void* out, int N, int C, int incoming, float eps, int stages,
+                           hipStream_t stream);
+
 // other pair widths (trimul_wide.hip; C = 256): same interface, blob layout in that file
 size_t trimul_wide_blob_bytes(int C);
 void trimul_wide_offsets(int C, size_t* gate, size_t* ab, size_t* out, size_t* ln, size_t* blk);
@@ -153,7 +163,7 @@ void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nba
 void launch_bias_tiles_f32(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
                            hipStream_t stream, int Lk = 0);
 
-enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS };
+enum : int { EPI_STORE = 0, EPI_SIGMOID, EPI_SWIGLU, EPI_ADALN, EPI_RESID, EPI_FRAG_CH, EPI_FRAG_POS, EPI_PLANES };
 
 // Rows are addressed as (a, position): a < rows_a, position < L, global row = a * L + position,
 // position blocks of 32 (nb = ceil(L / 32)).  Plain [M, K] problems use rows_a = 1, L = M.
@@ -175,6 +185,11 @@ struct LinearArgs {
     int parts;
     size_t a_part, w_part, out_part, aux_part;
     int gate_dtype;
+    // EPI_PLANES: out is bf16 channel-major planes [Nout][ldo][ldo], value (acc * sigmoid(acc2)) or 0
+    // where the position's mask byte is 0, stored at plane[c][a * ldo + position]; the mask byte of
+    // (a, position) is mask[a * L + position], or mask[position * rows_a + a] with mask_transposed.
+    // EPI_RESID: optional mask byte per output row (0 zeroes the row)
+    const uint8_t* mask; int mask_transposed;
 };
 int launch_linear(const LinearArgs& p, hipStream_t stream);
 

@@ -9,9 +9,11 @@
 //   EPI_SIGMOID  y = sigmoid(acc + bias)
 //   EPI_SWIGLU   y = silu(acc) * acc2                                    primitives/activation.py:27-29
 //   EPI_ADALN    y = sigmoid(acc + bias) * aux + acc2                    primitives/normalization.py:117-125
-//   EPI_RESID    y = aux + gate * (acc + bias)      (aux, gate optional) layers/folding/attention_pair_bias.py:155-157
+//   EPI_RESID    y = (aux + gate * (acc + bias)) * row mask   (aux, gate, mask optional)
+//                layers/folding/attention_pair_bias.py:155-157, modules/apo_module.py:172
 //   EPI_FRAG_CH  fragments with channels as accumulator rows (q, k, gate of attention)
 //   EPI_FRAG_POS fragments with positions as accumulator rows (v of attention)
+//   EPI_PLANES   (acc * sigmoid(acc2)) * mask as bf16 channel-major planes   primitives/triangle_multiplication.py:216-221
 #include "kernels.hpp"
 
 namespace kfh {
@@ -53,8 +55,8 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
     f32x16 acc, acc2;
 #pragma unroll
     for (int v = 0; v < 16; ++v) { acc[v] = 0.f; acc2[v] = 0.f; }
-    constexpr bool W_IS_A = (EPI == EPI_FRAG_CH);
-    constexpr bool TWO = (EPI == EPI_SWIGLU || EPI == EPI_ADALN);
+    constexpr bool W_IS_A = (EPI == EPI_FRAG_CH || EPI == EPI_PLANES);     // channels as accumulator rows
+    constexpr bool TWO = (EPI == EPI_SWIGLU || EPI == EPI_ADALN || EPI == EPI_PLANES);
     // part pairs (A part, W part) of one k-step, smallest terms first
     constexpr int NPROD = PARTS == 3 ? 6 : 1;
     constexpr int PA[6] = {PARTS == 3 ? 2 : 0, PARTS == 3 ? 1 : 0, 0, PARTS == 3 ? 1 : 0, 0, 0};
@@ -80,7 +82,7 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
             for (int pr = 0; pr < NPROD; ++pr) {
                 const bf16x8 xq = x[i][PA[pr]], wq = w[i][PW[pr]];
                 acc = W_IS_A ? mfma32(wq, xq, acc) : mfma32(xq, wq, acc);
-                if constexpr (TWO) acc2 = mfma32(xq, v[i][PW[pr]], acc2);
+                if constexpr (TWO) acc2 = W_IS_A ? mfma32(v[i][PW[pr]], xq, acc2) : mfma32(xq, v[i][PW[pr]], acc2);
             }
     };
     const int nch = ksteps / CH;
@@ -102,7 +104,10 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
                 const bf16x8 x = afrag(ks, PA[pr]);
                 const bf16x8 w = wfrag(Wb, ks, PW[pr]);
                 acc = W_IS_A ? mfma32(w, x, acc) : mfma32(x, w, acc);
-                if constexpr (TWO) acc2 = mfma32(x, wfrag(W2b, ks, PW[pr]), acc2);
+                if constexpr (TWO) {
+                    const bf16x8 w2 = wfrag(W2b, ks, PW[pr]);
+                    acc2 = W_IS_A ? mfma32(w2, x, acc2) : mfma32(x, w2, acc2);
+                }
             }
         }
     }
@@ -124,7 +129,23 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
             if constexpr (TWO) acc2[v] += red[w][1][v * 64 + lane];
         }
 
-    if constexpr (EPI == EPI_FRAG_CH || EPI == EPI_FRAG_POS) {
+    if constexpr (EPI == EPI_PLANES) {
+        // lane col <-> position, registers <-> 16 of the block's 32 channels: for one register the
+        // 32 lanes of a half write 32 consecutive positions of one plane
+        const int ps = blk * 32 + col;
+        if (ps >= p.L) return;
+        const size_t mi = p.mask_transposed ? (size_t)ps * p.rows_a + a : (size_t)a * p.L + ps;
+        const bool valid = p.mask[mi] != 0;
+        const size_t plane_sz = (size_t)p.ldo * p.ldo;
+        uint16_t* dst = static_cast<uint16_t*>(p.out) + (size_t)a * p.ldo + ps;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int c = 32 * wb + acc_row(v, half);
+            if (c >= p.Nout) continue;
+            const float y = valid ? acc[v] * sigmoidf_fast(acc2[v]) : 0.f;
+            dst[(size_t)c * plane_sz] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
+        }
+    } else if constexpr (EPI == EPI_FRAG_CH || EPI == EPI_FRAG_POS) {
         const int h = wb / p.PB, pp = wb % p.PB;
         if constexpr (EPI == EPI_FRAG_CH) {
 #pragma unroll
@@ -196,6 +217,7 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
                     y += p.aux_dtype == KFH_F32 ? static_cast<const float*>(p.aux)[r_aux * p.ld_aux + c]
                                                 : bf16_lo(static_cast<const uint16_t*>(p.aux)[r_aux * p.ld_aux + c]);
                 }
+                if (p.mask && p.mask[r] == 0) y = 0.f;       // row mask of the output (the block's final z * mask)
             }
             if (p.out_dtype == KFH_F32) {
                 static_cast<float*>(p.out)[r * p.ldo + c] = y;
@@ -237,6 +259,7 @@ int launch_linear(const LinearArgs& p, hipStream_t stream) {
         case EPI_RESID: if (p.a_frag) KFH_LIN(EPI_RESID, true, 1); else KFH_LIN(EPI_RESID, false, 1); break;
         case EPI_FRAG_CH: KFH_LIN(EPI_FRAG_CH, false, 1); break;
         case EPI_FRAG_POS: KFH_LIN(EPI_FRAG_POS, false, 1); break;
+        case EPI_PLANES: if (!p.mask || !p.W2) return -1; KFH_LIN(EPI_PLANES, false, 1); break;
         default: return -1;
     }
 #undef KFH_LIN

@@ -102,7 +102,7 @@ def trimul_pack(ln_in_w, ln_in_b, p_in_w, g_in_w, ln_out_w, ln_out_b, p_out_w, g
     C = p_out_w.shape[0]
     nbytes = L.kfh_trimul_packed_bytes(C)
     if nbytes == 0:
-        raise NotImplementedError(f"hip triangle multiplication is built for C=128, got {C}")
+        raise NotImplementedError(f"hip triangle multiplication takes C a multiple of 32 up to 256, got {C}")
     ws = _weights_f32(device, ln_in_w, ln_in_b, p_in_w, g_in_w, ln_out_w, ln_out_b, p_out_w, g_out_w)
     blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
@@ -144,7 +144,7 @@ def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, dire
     L = _lib.lib()
     ws_bytes = L.kfh_trimul_workspace_bytes(N, C)
     if ws_bytes == 0:
-        raise NotImplementedError(f"hip triangle multiplication is built for C=128 and C=256, got {C}")
+        raise NotImplementedError(f"hip triangle multiplication takes C a multiple of 32 up to 256, got {C}")
     ws = _workspace(workspace, ws_bytes, dev)
     d = KFH_INCOMING if direction == "incoming" else KFH_OUTGOING
     with torch.cuda.device(dev):

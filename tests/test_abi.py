@@ -30,7 +30,7 @@ def test_size_queries_and_argument_errors_need_no_gpu():
     from kfold_amd import _lib
 
     lib = _lib.lib()
-    assert lib.kfh_trimul_packed_bytes(128) > 0 and lib.kfh_trimul_packed_bytes(64) == 0
+    assert lib.kfh_trimul_packed_bytes(128) > 0 and lib.kfh_trimul_packed_bytes(64) > 0 and lib.kfh_trimul_packed_bytes(48) == 0
     assert lib.kfh_trimul_packed_bytes(256) > lib.kfh_trimul_packed_bytes(128)
     assert lib.kfh_triattn_packed_bytes(128, 4) > 0 and lib.kfh_triattn_packed_bytes(128, 3) == 0
     assert lib.kfh_triattn_packed_bytes(64, 4) > 0 and lib.kfh_triattn_packed_bytes(128, 1) == 0   # head dim > 64
@@ -41,8 +41,8 @@ def test_size_queries_and_argument_errors_need_no_gpu():
     assert lib.kfh_transition_workspace_bytes(1000, 384, 4) > 0
     assert lib.kfh_apb_packed_bytes(384, 16, 0, 0) > 0 and lib.kfh_apb_packed_bytes(384, 5, 0, 0) == 0
     # argument checks run before any GPU call
-    rc = lib.kfh_trimul_forward(None, None, None, None, None, None, 0, 1, 8, 64, 0, 1e-5, 0, None)
-    assert rc == -2 and b"C=64" in lib.kfh_last_error()
+    rc = lib.kfh_trimul_forward(None, None, None, None, None, None, 0, 1, 8, 48, 0, 1e-5, 0, None)
+    assert rc == -2 and b"C=48" in lib.kfh_last_error()
     rc = lib.kfh_trimul_forward(None, None, None, None, None, None, 0, 1, 8, 128, 0, 1e-5, 0, None)
     assert rc == -1 and b"null" in lib.kfh_last_error()
     rc = lib.kfh_triattn_forward(None, None, None, None, None, None, 0, 1, 9000, 128, 4, 0, 1e-5, 0, None)
@@ -246,10 +246,10 @@ def test_header_is_plain_c_and_a_c_caller_links(tmp_path):
 #include <string.h>
 int main(void) {
     if (kfh_version() < 1) return 1;
-    if (kfh_trimul_packed_bytes(128) == 0 || kfh_trimul_packed_bytes(64) != 0) return 2;
+    if (kfh_trimul_packed_bytes(128) == 0 || kfh_trimul_packed_bytes(48) != 0) return 2;
     if (kfh_transition_static_scratch_bytes() != (size_t)8 << 20) return 3;
-    int rc = kfh_trimul_forward(0, 0, 0, 0, 0, 0, 0, 1, 8, 64, KFH_OUTGOING, 1e-5f, KFH_BF16, 0);
-    if (rc != KFH_EUNSUPPORTED || !strstr(kfh_last_error(), "C=64")) return 4;
+    int rc = kfh_trimul_forward(0, 0, 0, 0, 0, 0, 0, 1, 8, 48, KFH_OUTGOING, 1e-5f, KFH_BF16, 0);
+    if (rc != KFH_EUNSUPPORTED || !strstr(kfh_last_error(), "C=48")) return 4;
     rc = kfh_trimul_forward(0, 0, 0, 0, 0, 0, 0, 1, 8, 128, KFH_OUTGOING, 1e-5f, KFH_BF16, 0);
     if (rc != KFH_EINVAL) return 5;
     printf("ok\n");

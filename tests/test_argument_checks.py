@@ -37,7 +37,7 @@ def test_trimul_argument_checks(env):
     lib, p, _ = env
     need = lib.kfh_trimul_workspace_bytes(64, 128)
     f = lib.kfh_trimul_forward
-    _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], need, 1, 64, 96, 0, 1e-5, 0, None), EUNSUPPORTED, "C=96")
+    _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], need, 1, 64, 80, 0, 1e-5, 0, None), EUNSUPPORTED, "C=80")
     _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], need, 0, 64, 128, 0, 1e-5, 0, None), EINVAL, "B=0")
     _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], need, 1, -3, 128, 0, 1e-5, 0, None), EINVAL, "N=-3")
     _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], need, 1, 64, 128, 0, 1e-5, 7, None), EINVAL, "io_dtype 7")
@@ -51,7 +51,7 @@ def test_trimul_argument_checks(env):
             "workspace", str(need))
     _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], 0, 1, 64, 256, 1, 1e-5, 1, None), EINVAL, "workspace")
     g = lib.kfh_trimul_pack
-    _expect(lib, g(*p[:8], 0, 64, p[8], None), EUNSUPPORTED, "C=64")
+    _expect(lib, g(*p[:8], 0, 48, p[8], None), EUNSUPPORTED, "C=48")
     _expect(lib, g(*p[:8], 5, 128, p[8], None), EINVAL, "w_dtype 5")
     _expect(lib, g(*p[:7], None, 0, 128, p[8], None), EINVAL, "null")
     _expect(lib, g(*p[:8], 0, 128, None, None), EINVAL, "null")
@@ -89,9 +89,9 @@ def test_transition_and_bias_argument_checks(env):
     _expect(lib, f(p[0], p[1], None, None, p[2], None, 0, -1, 128, 2, 1e-5, 0, None), EINVAL, "rows=-1")
     _expect(lib, f(p[0], p[1], None, None, p[2], None, 0, 10, 128, 2, 1e-5, 4, None), EINVAL, "io_dtype")
     _expect(lib, f(None, p[1], None, None, p[2], None, 0, 10, 128, 2, 1e-5, 0, None), EINVAL, "null")
-    # token-track widths: the row mask exists for the fused C=128 kernel only, the workspace is needed
-    _expect(lib, f(p[0], p[1], None, p[3], p[2], p[4], 1 << 30, 10, 384, 4, 1e-5, 0, None), EUNSUPPORTED, "mask")
+    # token-track widths need the workspace (the fused C = 128 / 256 kernels do not)
     need = lib.kfh_transition_workspace_bytes(10, 384, 4)
+    assert lib.kfh_transition_workspace_bytes(10, 256, 4) == 0 and lib.kfh_transition_workspace_bytes(10, 64, 2) > 0
     _expect(lib, f(p[0], p[1], None, None, p[2], p[4], need - 1, 10, 384, 4, 1e-5, 0, None), EINVAL, "workspace")
     _expect(lib, f(p[0], p[1], None, None, p[2], None, 0, 10, 384, 4, 1e-5, 0, None), EINVAL)
     g = lib.kfh_transition_pack

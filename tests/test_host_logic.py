@@ -138,7 +138,7 @@ def test_caller_workspace_is_used_and_checked(rec):
     need_tm = ops.workspace_bytes("trimul", N=N, C=128)
     need_ta = ops.workspace_bytes("triattn", N=N, C=128, heads=4)
     assert need_tm > 0 and need_ta > 0
-    assert ops.workspace_bytes("trimul", N=N, C=64) == 0
+    assert ops.workspace_bytes("trimul", N=N, C=48) == 0 and ops.workspace_bytes("trimul", N=N, C=64) > 0
     with pytest.raises(ValueError):
         ops.workspace_bytes("softmax", N=N)
     blob = torch.zeros(16, dtype=torch.uint8)
@@ -176,7 +176,7 @@ def test_wrappers_refuse_inconsistent_arguments_before_any_call(rec):
     with pytest.raises(ValueError, match="residual must"):
         ops.triattn_forward(z, m, blob, 4, True, residual=z.float())
     with pytest.raises(NotImplementedError):
-        ops.trimul_forward(torch.zeros(1, 8, 8, 64, dtype=torch.bfloat16), m, blob, "outgoing")
+        ops.trimul_forward(torch.zeros(1, 8, 8, 48, dtype=torch.bfloat16), m, blob, "outgoing")
     with pytest.raises(TypeError, match="bfloat16 and float32"):
         ops.trimul_forward(z.half(), m, blob, "outgoing")
     assert rec.names() == []
@@ -270,8 +270,9 @@ def test_other_widths_take_the_generic_entry_points(rec):
     with torch.no_grad():
         primitives.TriangleMultiplicationIncoming(256).eval()(torch.zeros(2, 8, 8, 256, dtype=torch.bfloat16), m)
         primitives.TriangleAttentionEndingNode(64, 4).eval()(torch.zeros(2, 8, 8, 64, dtype=torch.bfloat16), m)
-        with pytest.raises(NotImplementedError):
-            primitives.TriangleMultiplicationIncoming(64).eval()(torch.zeros(2, 8, 8, 64, dtype=torch.bfloat16), m)
+        primitives.TriangleMultiplicationIncoming(64).eval()(torch.zeros(2, 8, 8, 64, dtype=torch.bfloat16), m)
+        with pytest.raises(NotImplementedError):     # not a multiple of 32
+            primitives.TriangleMultiplicationIncoming(48).eval()(torch.zeros(2, 8, 8, 48, dtype=torch.bfloat16), m)
     tm = rec.of("kfh_trimul_forward")[0]
     assert tm[7:11] == (2, 8, 256, 1)
     ta = rec.of("kfh_triattn_forward")[0]

@@ -83,6 +83,21 @@ def test_walk_triattn_c64_templates(n, batch):
             mod(x, arena.like(pm))
 
 
+def test_walk_template_stack_block_c64():
+    """The apo template stack's Pairformer block: c = 64 (tri-mul and transition through the paths
+    assembled from the token-track kernels), 4 templates of 384 tokens."""
+    from kfold_amd import modules as M
+
+    n, batch = 384, 4
+    blk = M.PairformerBlock(64, 4).eval()
+    synthetic.init_weights_(blk, 4)
+    tok = synthetic.token_mask(n, synthetic.n_pad_for(n, 0.1))
+    pm = synthetic.pair_mask_from_tokens(tok).expand(batch, n, n).contiguous()
+    with torch.no_grad(), _walk(stride=307) as arena:
+        z = arena.like(_pattern((batch, n, n, 64)))
+        blk(z, arena.like(pm), inplace_output=True)
+
+
 def test_walk_diffusion_attention_and_windows():
     """Diffusion-transformer pair-bias attention (5 samples, one bias, 768 tokens, 16 x 48) and
     the local cross-attention windows (32 queries x 128 keys)."""

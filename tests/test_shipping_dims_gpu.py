@@ -176,3 +176,66 @@ def test_triattn_c64_templates_n384(starting):
             want = ref.mha(xn[:, rows], xn[:, rows], bias, mt[..., :, None, None, :][:, rows])[0]
             gb = (got[b] if starting else got[b].transpose(0, 1))[rows]
             print(assert_close(gb, want, f"triattn c=64 template {b}", auto_scale=True), flush=True)
+
+
+@pytest.mark.parametrize("direction", ["outgoing", "incoming"])
+@pytest.mark.parametrize("c,n,n_pad", [(64, 37, 5), (64, 70, 0), (96, 50, 6)])
+def test_trimul_other_widths(direction, c, n, n_pad):
+    """Triangle multiplication at the template stack's width (c = 64) and at another multiple of
+    32: the path assembled from the token-track kernels and the contraction kernel."""
+    from kfold_amd import ops, primitives as P
+    from oracle import torch_path as O
+
+    print(f"case trimul C={c} {direction} n={n}", flush=True)
+    cls = "TriangleMultiplicationOutgoing" if direction == "outgoing" else "TriangleMultiplicationIncoming"
+    ref = getattr(O, cls)(c).eval()
+    synthetic.init_weights_(ref, 3, std=0.05)
+    _affine(ref)
+    hip = getattr(P, cls)(c).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    z, _, pm = synthetic.pair_inputs(n, c, n_pad, seed=n)
+    if n == 70:         # a general (not outer-product) mask
+        pm = torch.rand(1, n, n, generator=torch.Generator().manual_seed(5)) > 0.3
+    zb = z.bfloat16()
+    with torch.no_grad():
+        want = ref(zb.float(), pm)
+        zd, pmd = zb.to(DEV), pm.to(DEV)
+        got = hip(zd, pmd)
+        print(assert_close(got, want, f"trimul C={c} {direction}", auto_scale=True), flush=True)
+        assert torch.equal(got, hip(zd, pmd)), "run-to-run results differ"
+        zin = zd.clone()
+        ops.trimul_forward(zin, pmd, hip._hip_multiplication_cache, direction, residual=zin, out=zin)
+        assert_close(zin, zb.float() + want, "residual in place", rel_fro=5e-3, auto_scale=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_template_stack_block_c64(dtype):
+    """The whole Pairformer block of the apo template stack (model/modules/apo_module.py:107-172,
+    :294-301: channel_z = 64, 4 triangle-attention heads of 16) over a batch of templates, in place,
+    with the final mask."""
+    from kfold_amd import modules as M
+    from oracle import torch_path as O
+
+    print(f"case template-stack block C=64 {dtype}", flush=True)
+    ref = O.PairformerBlock(64, 4).eval()
+    synthetic.init_weights_(ref, 21, std=0.05)
+    hip = M.PairformerBlock(64, 4).eval()
+    hip.load_state_dict(ref.state_dict())
+    hip.to(DEV)
+    n, batch = 44, 3
+    g = torch.Generator().manual_seed(4)
+    z = torch.randn(batch, n, n, 64, generator=g)
+    pm = torch.stack([synthetic.pair_mask_from_tokens(synthetic.token_mask(n, pad))[0] for pad in (0, 5, 12)])
+    zi = z.to(dtype)
+    with torch.no_grad():
+        zw = torch.stack([ref(zi[b:b + 1].float().clone(), pm[b:b + 1].float())[0] for b in range(batch)])
+        zin = zi.to(DEV)
+        zg = hip(zin, pm.to(DEV), inplace_output=True)
+    assert zg.data_ptr() == zin.data_ptr()
+    if dtype == torch.float32:
+        print(assert_close(zg, zw, "template-stack block, fp32 stream", rel_fro=5e-3, auto_scale=True), flush=True)
+    else:   # bf16 stream: five storage roundings of |z| up to ~5 on top of the kernel error
+        print(assert_close(zg, zw, "template-stack block, bf16 stream", max_abs=8e-2, mean_abs=6e-3, rel_fro=8e-3),
+              flush=True)
+    assert (zg.cpu()[~pm] == 0).all()
