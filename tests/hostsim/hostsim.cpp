@@ -94,6 +94,7 @@ Lane* cur() { return t_cur; }
 char* dynamic_lds() { return t_worker->lds; }
 
 static std::atomic<int> g_skip_math{0};
+static std::atomic<int> g_schedule{0};      // order in which runnable lanes are resumed (see hostsim_set_schedule)
 static std::atomic<int> g_fill{1};
 
 [[noreturn]] static void die(const char* what) {
@@ -208,9 +209,18 @@ static void run_block(Worker* wk, dim3 grid, dim3 block, dim3 bidx) {
         f.sp = sp;
     }
     int remaining = nt;
+    const int schedule = g_schedule.load(std::memory_order_relaxed);
+    unsigned pass = 0;
     while (remaining > 0) {
         bool progress = false;
-        for (int t = 0; t < nt; ++t) {
+        ++pass;
+        for (int k = 0; k < nt; ++k) {
+            // 0: lanes in order; 1: in reverse; 2: wavefronts in an order that rotates from pass to
+            // pass.  A kernel free of races between wavefronts gives the same bits under all three.
+            int t = k;
+            if (schedule == 1) t = nt - 1 - k;
+            else if (schedule == 2) t = (int)((((k >> 6) + pass * 7) % (unsigned)nw) << 6 | (k & 63));
+            if (t >= nt) continue;
             Fiber& f = wk->fibers[t];
             if (f.done) continue;
             if (f.wait_kind == 1 && f.lane.wave->gen == f.wait_gen) continue;
@@ -466,6 +476,9 @@ void hostsim_set_block_filter(long long stride, long long edge) {
 
 // 1 (default): new buffers are filled with 0xFF; 0: left as the zero pages the kernel maps
 void hostsim_set_fill(int on) { hostsim::g_fill.store(on); }
+// Order in which the lanes of a workgroup are resumed: 0 ascending, 1 descending, 2 wavefronts
+// rotating.  Results of a correctly synchronised kernel do not depend on it.
+void hostsim_set_schedule(int mode) { hostsim::g_schedule.store(mode); }
 void hostsim_set_skip_math(int on) { hostsim::g_skip_math.store(on); }
 // per-kernel launch counts and host seconds since the last call, to stderr
 void hostsim_report(void) {
