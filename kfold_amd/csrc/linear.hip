@@ -14,9 +14,123 @@
 //   EPI_FRAG_CH  fragments with channels as accumulator rows (q, k, gate of attention)
 //   EPI_FRAG_POS fragments with positions as accumulator rows (v of attention)
 //   EPI_PLANES   (acc * sigmoid(acc2)) * mask as bf16 channel-major planes   primitives/triangle_multiplication.py:216-221
+#include <cstdlib>
+
 #include "kernels.hpp"
 
 namespace kfh {
+
+// Epilogue of one 32 x 32 accumulator block: `a` = row group, `blk` = position block inside it,
+// `wb` = 32-channel block of the packed weight.  Shared by the two kernels below.
+template <int EPI, int PARTS>
+__device__ __forceinline__ void linear_epilogue(const LinearArgs& p, f32x16& acc, f32x16& acc2, int a, int blk,
+                                                int wb, int lane) {
+    const int col = lane & 31, half = lane >> 5;
+    if constexpr (EPI == EPI_PLANES) {
+        // lane col <-> position, registers <-> 16 of the block's 32 channels: for one register the
+        // 32 lanes of a half write 32 consecutive positions of one plane
+        const int ps = blk * 32 + col;
+        if (ps >= p.L) return;
+        const size_t mi = p.mask_transposed ? (size_t)ps * p.rows_a + a : (size_t)a * p.L + ps;
+        const bool valid = p.mask[mi] != 0;
+        const size_t plane_sz = (size_t)p.ldo * p.ldo;
+        uint16_t* dst = static_cast<uint16_t*>(p.out) + (size_t)a * p.ldo + ps;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int c = 32 * wb + acc_row(v, half);
+            if (c >= p.Nout) continue;
+            const float y = valid ? acc[v] * sigmoidf_fast(acc2[v]) : 0.f;
+            dst[(size_t)c * plane_sz] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
+        }
+    } else if constexpr (EPI == EPI_FRAG_CH || EPI == EPI_FRAG_POS) {
+        const int h = wb / p.PB, pp = wb % p.PB;
+        if constexpr (EPI == EPI_FRAG_CH) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int d = 32 * pp + acc_row(v, half);
+                float y = acc[v];
+                if (p.bias && d < p.Dh) y += p.bias[h * p.Dh + d] * p.bias_scale;
+                if (p.sigmoid) y = PARTS == 3 ? 1.0f / (1.0f + exp2f(-kLog2e * y)) : sigmoidf_fast(y);
+                acc[v] = y;
+            }
+        }
+        const size_t u0 = (((((size_t)a * p.H + h) * p.nb + blk) * p.PB + pp) * 2 * 64 + lane) * 16;
+        if constexpr (PARTS == 1) {
+            bf16x8 f0, f1;
+            acc_to_frags(acc, f0, f1);
+            bf16x8* dst = reinterpret_cast<bf16x8*>(static_cast<char*>(p.out) + u0);
+            dst[0] = f0;
+            dst[64] = f1;
+        } else {
+            f32x16 part[PARTS];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                float sp[3];
+                split3(acc[v], sp);
+#pragma unroll
+                for (int q = 0; q < PARTS; ++q) part[q][v] = sp[q];
+            }
+#pragma unroll
+            for (int q = 0; q < PARTS; ++q) {
+                bf16x8 f0, f1;
+                acc_to_frags(part[q], f0, f1);
+                bf16x8* dst = reinterpret_cast<bf16x8*>(static_cast<char*>(p.out) + (size_t)q * p.out_part + u0);
+                dst[0] = f0;
+                dst[64] = f1;
+            }
+        }
+    } else {
+        const int c = 32 * wb + col;
+        if (c >= p.Nout) return;
+        const float bc = p.bias ? p.bias[c] : 0.f;
+        auto sig = [&](float x) { return PARTS == 3 ? 1.0f / (1.0f + exp2f(-kLog2e * x)) : sigmoidf_fast(x); };
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int ps = blk * 32 + acc_row(v, half);
+            if (ps >= p.L) continue;
+            size_t r = (size_t)a * p.L + ps;
+            size_t r_aux = (size_t)(p.aux_shared ? 0 : a) * p.L + ps;
+            if constexpr (EPI == EPI_RESID) {
+                if (p.out_transposed) { r = (size_t)ps * p.rows_a + a; r_aux = r; }
+            }
+            const size_t r_gate = (size_t)(p.gate_shared ? 0 : a) * p.L + ps;
+            float y = acc[v] + bc;
+            if constexpr (EPI == EPI_SIGMOID) y = sig(y);
+            if constexpr (EPI == EPI_SWIGLU) y = acc[v] * sig(acc[v]) * acc2[v];
+            if constexpr (EPI == EPI_ADALN) {
+                const char* ap = static_cast<const char*>(p.aux) + (r_aux * p.ld_aux + c) * 2;
+                float ax = bf16_lo(*reinterpret_cast<const uint16_t*>(ap));
+                if constexpr (PARTS == 3)
+                    ax = (bf16_lo(*reinterpret_cast<const uint16_t*>(ap + 2 * p.aux_part)) +
+                          bf16_lo(*reinterpret_cast<const uint16_t*>(ap + p.aux_part))) + ax;
+                y = sig(y) * ax + acc2[v];
+            }
+            if constexpr (EPI == EPI_RESID) {
+                if (p.gate) {
+                    y *= p.gate_dtype == KFH_F32 ? reinterpret_cast<const float*>(p.gate)[r_gate * p.ld_gate + c]
+                                                 : bf16_lo(p.gate[r_gate * p.ld_gate + c]);
+                }
+                if (p.aux) {
+                    y += p.aux_dtype == KFH_F32 ? static_cast<const float*>(p.aux)[r_aux * p.ld_aux + c]
+                                                : bf16_lo(static_cast<const uint16_t*>(p.aux)[r_aux * p.ld_aux + c]);
+                }
+                if (p.mask && p.mask[r] == 0) y = 0.f;       // row mask of the output (the block's final z * mask)
+            }
+            if (p.out_dtype == KFH_F32) {
+                static_cast<float*>(p.out)[r * p.ldo + c] = y;
+            } else if constexpr (PARTS == 1) {
+                static_cast<uint16_t*>(p.out)[r * p.ldo + c] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
+            } else {
+                float sp[3];
+                split3(y, sp);
+#pragma unroll
+                for (int q = 0; q < PARTS; ++q)
+                    *reinterpret_cast<uint16_t*>(static_cast<char*>(p.out) + (size_t)q * p.out_part + (r * p.ldo + c) * 2) =
+                        (uint16_t)(pack_bf16(sp[q], 0.f) & 0xffffu);
+            }
+        }
+    }
+}
 
 // PARTS = 3 is the fp32 arithmetic: A, W (and W2) arrive as their three split3 planes and every
 // k-step runs the six part products (i, j), i + j <= 2; bf16 outputs leave as three planes too.
@@ -129,110 +243,107 @@ __global__ __launch_bounds__(256) void linear_kernel(LinearArgs p) {
             if constexpr (TWO) acc2[v] += red[w][1][v * 64 + lane];
         }
 
-    if constexpr (EPI == EPI_PLANES) {
-        // lane col <-> position, registers <-> 16 of the block's 32 channels: for one register the
-        // 32 lanes of a half write 32 consecutive positions of one plane
-        const int ps = blk * 32 + col;
-        if (ps >= p.L) return;
-        const size_t mi = p.mask_transposed ? (size_t)ps * p.rows_a + a : (size_t)a * p.L + ps;
-        const bool valid = p.mask[mi] != 0;
-        const size_t plane_sz = (size_t)p.ldo * p.ldo;
-        uint16_t* dst = static_cast<uint16_t*>(p.out) + (size_t)a * p.ldo + ps;
+    linear_epilogue<EPI, PARTS>(p, acc, acc2, a, blk, wb, lane);
+}
+
+// The same products for problems with many rows (the diffusion attention's 5 x 768 tokens, the
+// N^2 positions of the generic pair-track paths): one workgroup computes 128 positions x 128 output
+// channels, its 4 wavefronts in a 2 x 2 grid of 64 x 64 (2 position blocks x 2 weight blocks, every
+// fragment feeds two MFMAs), the whole K per wavefront in register-prefetched chunks, no partial sums.
+template <int EPI, bool AFRAG>
+__global__ __launch_bounds__(256) void linear_tile_kernel(LinearArgs p) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, half = lane >> 5;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int groups = (p.nb + 3) / 4;                       // groups of 4 position blocks per row group
+    const int a = blockIdx.x / groups, blk0 = (blockIdx.x % groups) * 4 + 2 * wm;
+    const int wb0 = blockIdx.y * 4 + 2 * wn;
+    const int ksteps = p.K / 16;
+    constexpr bool W_IS_A = (EPI == EPI_FRAG_CH || EPI == EPI_PLANES);
+    constexpr bool TWO = (EPI == EPI_SWIGLU || EPI == EPI_ADALN || EPI == EPI_PLANES);
+    constexpr int CH = TWO ? 2 : 4;                          // k-steps per prefetched chunk
+
+    // blocks past the end are clamped for the loads and skipped in the epilogue
+    int blk[2], wb[2];
+    const char* arow[2];
+    const char* Wb[2];
+    const char* W2b[2];
+    const int dks = 2 * p.PB;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int c = 32 * wb + acc_row(v, half);
-            if (c >= p.Nout) continue;
-            const float y = valid ? acc[v] * sigmoidf_fast(acc2[v]) : 0.f;
-            dst[(size_t)c * plane_sz] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
-        }
-    } else if constexpr (EPI == EPI_FRAG_CH || EPI == EPI_FRAG_POS) {
-        const int h = wb / p.PB, pp = wb % p.PB;
-        if constexpr (EPI == EPI_FRAG_CH) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int d = 32 * pp + acc_row(v, half);
-                float y = acc[v];
-                if (p.bias && d < p.Dh) y += p.bias[h * p.Dh + d] * p.bias_scale;
-                if (p.sigmoid) y = PARTS == 3 ? 1.0f / (1.0f + exp2f(-kLog2e * y)) : sigmoidf_fast(y);
-                acc[v] = y;
-            }
-        }
-        const size_t u0 = (((((size_t)a * p.H + h) * p.nb + blk) * p.PB + pp) * 2 * 64 + lane) * 16;
-        if constexpr (PARTS == 1) {
-            bf16x8 f0, f1;
-            acc_to_frags(acc, f0, f1);
-            bf16x8* dst = reinterpret_cast<bf16x8*>(static_cast<char*>(p.out) + u0);
-            dst[0] = f0;
-            dst[64] = f1;
+    for (int i = 0; i < 2; ++i) {
+        blk[i] = min(blk0 + i, p.nb - 1);
+        wb[i] = min(wb0 + i, p.nblk - 1);
+        const int pos = min(blk[i] * 32 + col, p.L - 1);
+        arow[i] = AFRAG ? nullptr
+                        : static_cast<const char*>(p.A) +
+                              (((size_t)(p.a_shared ? 0 : a) * p.L + pos) * p.lda + 8 * half) * 2;
+        Wb[i] = static_cast<const char*>(p.W) + ((size_t)wb[i] * ksteps * 64 + lane) * 16;
+        W2b[i] = p.W2 ? static_cast<const char*>(p.W2) + ((size_t)wb[i] * ksteps * 64 + lane) * 16 : nullptr;
+    }
+    auto afrag = [&](int i, int ks) -> bf16x8 {
+        if constexpr (AFRAG) {
+            const int h = ks / dks, kk = ks % dks;
+            const size_t u = ((((size_t)a * p.H + h) * p.nb + blk[i]) * dks + kk) * 64 + lane;
+            return *reinterpret_cast<const bf16x8*>(static_cast<const char*>(p.A) + u * 16);
         } else {
-            f32x16 part[PARTS];
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float sp[3];
-                split3(acc[v], sp);
-#pragma unroll
-                for (int q = 0; q < PARTS; ++q) part[q][v] = sp[q];
-            }
-#pragma unroll
-            for (int q = 0; q < PARTS; ++q) {
-                bf16x8 f0, f1;
-                acc_to_frags(part[q], f0, f1);
-                bf16x8* dst = reinterpret_cast<bf16x8*>(static_cast<char*>(p.out) + (size_t)q * p.out_part + u0);
-                dst[0] = f0;
-                dst[64] = f1;
-            }
+            return *reinterpret_cast<const bf16x8*>(arow[i] + 32 * ks);
         }
-    } else {
-        const int c = 32 * wb + col;
-        if (c >= p.Nout) return;
-        const float bc = p.bias ? p.bias[c] : 0.f;
-        auto sig = [&](float x) { return PARTS == 3 ? 1.0f / (1.0f + exp2f(-kLog2e * x)) : sigmoidf_fast(x); };
+    };
+    auto wfrag = [&](const char* base, int ks) -> bf16x8 {
+        return *reinterpret_cast<const bf16x8*>(base + (size_t)ks * 1024);
+    };
+
+    f32x16 acc[2][2], acc2[2][2];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int ps = blk * 32 + acc_row(v, half);
-            if (ps >= p.L) continue;
-            size_t r = (size_t)a * p.L + ps;
-            size_t r_aux = (size_t)(p.aux_shared ? 0 : a) * p.L + ps;
-            if constexpr (EPI == EPI_RESID) {
-                if (p.out_transposed) { r = (size_t)ps * p.rows_a + a; r_aux = r; }
-            }
-            const size_t r_gate = (size_t)(p.gate_shared ? 0 : a) * p.L + ps;
-            float y = acc[v] + bc;
-            if constexpr (EPI == EPI_SIGMOID) y = sig(y);
-            if constexpr (EPI == EPI_SWIGLU) y = acc[v] * sig(acc[v]) * acc2[v];
-            if constexpr (EPI == EPI_ADALN) {
-                const char* ap = static_cast<const char*>(p.aux) + (r_aux * p.ld_aux + c) * 2;
-                float ax = bf16_lo(*reinterpret_cast<const uint16_t*>(ap));
-                if constexpr (PARTS == 3)
-                    ax = (bf16_lo(*reinterpret_cast<const uint16_t*>(ap + 2 * p.aux_part)) +
-                          bf16_lo(*reinterpret_cast<const uint16_t*>(ap + p.aux_part))) + ax;
-                y = sig(y) * ax + acc2[v];
-            }
-            if constexpr (EPI == EPI_RESID) {
-                if (p.gate) {
-                    y *= p.gate_dtype == KFH_F32 ? reinterpret_cast<const float*>(p.gate)[r_gate * p.ld_gate + c]
-                                                 : bf16_lo(p.gate[r_gate * p.ld_gate + c]);
-                }
-                if (p.aux) {
-                    y += p.aux_dtype == KFH_F32 ? static_cast<const float*>(p.aux)[r_aux * p.ld_aux + c]
-                                                : bf16_lo(static_cast<const uint16_t*>(p.aux)[r_aux * p.ld_aux + c]);
-                }
-                if (p.mask && p.mask[r] == 0) y = 0.f;       // row mask of the output (the block's final z * mask)
-            }
-            if (p.out_dtype == KFH_F32) {
-                static_cast<float*>(p.out)[r * p.ldo + c] = y;
-            } else if constexpr (PARTS == 1) {
-                static_cast<uint16_t*>(p.out)[r * p.ldo + c] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
-            } else {
-                float sp[3];
-                split3(y, sp);
+    for (int m = 0; m < 2; ++m)
 #pragma unroll
-                for (int q = 0; q < PARTS; ++q)
-                    *reinterpret_cast<uint16_t*>(static_cast<char*>(p.out) + (size_t)q * p.out_part + (r * p.ldo + c) * 2) =
-                        (uint16_t)(pack_bf16(sp[q], 0.f) & 0xffffu);
+        for (int n = 0; n < 2; ++n)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) { acc[m][n][v] = 0.f; acc2[m][n][v] = 0.f; }
+
+    bf16x8 xa[CH][2], wa[CH][2], va[CH][2], xb[CH][2], wb2[CH][2], vb[CH][2];
+    auto load = [&](int c, bf16x8 (&x)[CH][2], bf16x8 (&w)[CH][2], bf16x8 (&v)[CH][2]) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int ks = min(c * CH + i, ksteps - 1);        // the last chunk may be short
+                x[i][j] = afrag(j, ks);
+                w[i][j] = wfrag(Wb[j], ks);
+                if constexpr (TWO) v[i][j] = wfrag(W2b[j], ks);
             }
+    };
+    auto compute = [&](int c, const bf16x8 (&x)[CH][2], const bf16x8 (&w)[CH][2], const bf16x8 (&v)[CH][2]) {
+#pragma unroll
+        for (int i = 0; i < CH; ++i) {
+            if (c * CH + i >= ksteps) break;
+#pragma unroll
+            for (int m = 0; m < 2; ++m)
+#pragma unroll
+                for (int n = 0; n < 2; ++n) {
+                    acc[m][n] = W_IS_A ? mfma32(w[i][n], x[i][m], acc[m][n]) : mfma32(x[i][m], w[i][n], acc[m][n]);
+                    if constexpr (TWO)
+                        acc2[m][n] = W_IS_A ? mfma32(v[i][n], x[i][m], acc2[m][n]) : mfma32(x[i][m], v[i][n], acc2[m][n]);
+                }
+        }
+    };
+    const int nch = (ksteps + CH - 1) / CH;
+    load(0, xa, wa, va);
+    for (int c = 0; c < nch; c += 2) {
+        if (c + 1 < nch) load(c + 1, xb, wb2, vb);
+        compute(c, xa, wa, va);
+        if (c + 1 < nch) {
+            if (c + 2 < nch) load(c + 2, xa, wa, va);
+            compute(c + 1, xb, wb2, vb);
         }
     }
+#pragma unroll
+    for (int m = 0; m < 2; ++m)
+#pragma unroll
+        for (int n = 0; n < 2; ++n) {
+            if (blk0 + m >= p.nb || wb0 + n >= p.nblk) continue;
+            linear_epilogue<EPI, 1>(p, acc[m][n], acc2[m][n], a, blk0 + m, wb0 + n, lane);
+        }
 }
 
 int launch_linear(const LinearArgs& p, hipStream_t stream) {
@@ -251,6 +362,30 @@ int launch_linear(const LinearArgs& p, hipStream_t stream) {
         return 0;
     }
     if (p.parts != 0 && p.parts != 1) return -1;
+    // many rows and more than one weight block: the 128 x 128 tile kernel, once its grid has enough
+    // workgroups for the chip (default 128; the environment variable KFH_LINEAR_TILE_MIN_WORKGROUPS
+    // overrides it, e.g. 1 to use the tile kernel wherever it applies)
+    const char* tile_env = std::getenv("KFH_LINEAR_TILE_MIN_WORKGROUPS");
+    const long long tile_req = tile_env ? std::atoll(tile_env) : 0;
+    const long long tile_min = tile_req > 0 ? tile_req : 128LL;
+    const long long tile_groups = (long long)p.rows_a * ((p.nb + 3) / 4);
+    const int tile_cols = (p.nblk + 3) / 4;
+    if (p.nblk >= 2 && tile_groups * tile_cols >= tile_min && tile_groups <= 0x7fffffffLL) {
+        dim3 tgrid((unsigned)tile_groups, (unsigned)tile_cols);
+#define KFH_TILE(E, F) hipLaunchKernelGGL((linear_tile_kernel<E, F>), tgrid, block, 0, stream, p)
+        switch (p.epi) {
+            case EPI_STORE: if (p.a_frag) KFH_TILE(EPI_STORE, true); else KFH_TILE(EPI_STORE, false); return 0;
+            case EPI_SIGMOID: KFH_TILE(EPI_SIGMOID, false); return 0;
+            case EPI_SWIGLU: KFH_TILE(EPI_SWIGLU, false); return 0;
+            case EPI_ADALN: KFH_TILE(EPI_ADALN, false); return 0;
+            case EPI_RESID: if (p.a_frag) KFH_TILE(EPI_RESID, true); else KFH_TILE(EPI_RESID, false); return 0;
+            case EPI_FRAG_CH: KFH_TILE(EPI_FRAG_CH, false); return 0;
+            case EPI_FRAG_POS: KFH_TILE(EPI_FRAG_POS, false); return 0;
+            case EPI_PLANES: if (!p.mask || !p.W2) return -1; KFH_TILE(EPI_PLANES, false); return 0;
+            default: return -1;
+        }
+#undef KFH_TILE
+    }
     switch (p.epi) {
         case EPI_STORE: if (p.a_frag) KFH_LIN(EPI_STORE, true, 1); else KFH_LIN(EPI_STORE, false, 1); break;
         case EPI_SIGMOID: KFH_LIN(EPI_SIGMOID, false, 1); break;

@@ -70,3 +70,29 @@ for _name in GPU_MODULES:
     for _attr, _fn in list(vars(_mod).items()):
         if _attr.startswith("test_") and callable(_fn) and _attr not in SKIP:
             globals()[f"test_host_{_short}__{_attr[5:]}"] = _twin(_mod, _fn)
+
+
+# The token-track linears pick between two kernels by problem size (one 32 x 32 tile per workgroup
+# with K split over its wavefronts, or 128 x 128 tiles): the unit-sized cases above mostly take the
+# first, so a selection of them runs again with the tile kernel forced wherever it applies.
+import tests.test_shipping_dims_gpu as _SD      # noqa: E402
+import tests.test_single_track_gpu as _ST       # noqa: E402
+
+_TILE_CASES = [
+    (_ST, "test_transition_parity", (384, 4, 70, torch.bfloat16)),
+    (_ST, "test_pair_bias_projection_and_trunk_apb", (96,)),
+    (_ST, "test_apb_functional_normalised_inputs_and_full_mask", ()),
+    (_ST, "test_apb_diffusion_variant", (False,)),
+    (_ST, "test_cross_attention_local_windows", (True,)),
+    (_SD, "test_triattn_other_widths_batched", (True, 64, 4, 50, 4)),
+    (_SD, "test_triattn_other_widths_batched", (False, 96, 2, 37, 2)),
+    (_SD, "test_trimul_other_widths", ("incoming", 64, 70, 0)),
+    (_SD, "test_template_stack_block_c64", (torch.float32,)),
+]
+
+
+@pytest.mark.parametrize("mod,name,args", _TILE_CASES, ids=[f"{n}{list(a)}" for _, n, a in _TILE_CASES])
+def test_host_tile_kernel_forced(mod, name, args, monkeypatch):
+    monkeypatch.setenv("KFH_LINEAR_TILE_MIN_WORKGROUPS", "1")
+    with _on_host(mod):
+        getattr(mod, name)(*args)
