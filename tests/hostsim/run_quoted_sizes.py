@@ -27,6 +27,7 @@ CASES = [
     (Q, "test_apb_diffusion_variant_n768", [(False,), (True,)]),
     (Q, "test_block_n768_metric_shape", [()]),
     (TA, "test_triattn_long_sequence_sampled_rows", [()]),
+    (TA, "test_triattn_config3_n512", [(True,), (False,)]),
     (SD, "test_triattn_c64_templates_n384", [(True,), (False,)]),
     (SD, "test_trimul_c256_tiled_sizes", [(384, "outgoing"), (384, "incoming"), (768, "outgoing"), (768, "incoming")]),
 ]

@@ -38,6 +38,8 @@ SKIP: dict[str, str] = {
     "test_cpu_tensors_are_rejected": "the twin runs on CPU tensors by design",
     "test_triattn_long_sequence_sampled_rows": "N = 1248 takes two minutes of CPU time "
                                                "(tests/hostsim/run_quoted_sizes.py runs it)",
+    "test_triattn_config3_n512": "benchmark config 3 at N = 512: a quarter of a minute of CPU time per node type "
+                                 "(tests/hostsim/run_quoted_sizes.py runs it; N = 256 and 130 stay here)",
     "test_triattn_c64_templates_n384": "4 templates at N = 384: half a minute of CPU time each "
                                        "(tests/hostsim/run_quoted_sizes.py runs them)",
     "test_trimul_c256_tiled_sizes": "N = 384 / 768 at C = 256: half a minute to minutes of CPU time each "
