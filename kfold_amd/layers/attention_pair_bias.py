@@ -59,7 +59,8 @@ def norm_eps(module: nn.Module) -> float:
     return module.layernorm_a.eps if hasattr(module, "layernorm_a") else 1e-5
 
 
-def select_arith(module: nn.Module, x: torch.Tensor) -> int:
+def select_arith(module: nn.Module, x: torch.Tensor, call_site: str | None = None) -> int:
+    """``call_site``: the one the caller names (the functional entry), else the module's own."""
     mode = getattr(module, "arith", "auto")
     if mode == "f32":
         return ops.KFH_ARITH_F32
@@ -67,7 +68,8 @@ def select_arith(module: nn.Module, x: torch.Tensor) -> int:
         return ops.KFH_ARITH_BF16
     if mode != "auto":
         raise ValueError(f"arith must be 'auto', 'bf16' or 'f32', got {mode!r}")
-    diffusion = str(getattr(module, "call_site", "diffusion_local")).startswith("diffusion")
+    site = call_site if call_site is not None else getattr(module, "call_site", "diffusion_local")
+    diffusion = str(site).startswith("diffusion")
     if diffusion and x.dtype == torch.float32 and not torch.is_autocast_enabled():
         return ops.KFH_ARITH_F32
     return ops.KFH_ARITH_BF16
@@ -82,14 +84,14 @@ def _flatten(t: torch.Tensor, keep: int, lead: torch.Size):
     return full.reshape((-1,) + t.shape[t.dim() - keep:]), True
 
 
-def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
+def _run(module, a, s, pair_bias, mask, apply_norm: bool, call_site: str | None = None) -> torch.Tensor:
     check_inference(a, "pair-bias attention")
     check_inf(module)
     if module.linear_g.bias is not None or module.linear_out.bias is not None:
         raise NotImplementedError("hip pair-bias attention: gate / output projection biases")
     params = _parameters(module)
     C, H, Cs = module.channel_a, module.num_heads, _cond_channels(module)
-    arith = select_arith(module, a)
+    arith = select_arith(module, a, call_site)
     key = cache_key(tuple(params.values()), a,
                     torch.float32 if arith == ops.KFH_ARITH_F32 else torch.bfloat16)
     blob = cached_blob(module, "_hip_apb_cache", key,
@@ -108,7 +110,7 @@ def _run(module, a, s, pair_bias, mask, apply_norm: bool) -> torch.Tensor:
     return out.reshape(a.shape).to(a.dtype)
 
 
-def _run_cross(module, x_q, x_k, pair_bias, mask) -> torch.Tensor:
+def _run_cross(module, x_q, x_k, pair_bias, mask, call_site: str | None = None) -> torch.Tensor:
     """Already normalised queries x_q [*, Lq, C] against keys x_k [*, Lk, C]: q/k/v/gate/output
     projections and the attention only (the caller has normalised and applies its own
     conditioning gate afterwards, attention_pair_bias.py:241-262 of the reference)."""
@@ -118,7 +120,7 @@ def _run_cross(module, x_q, x_k, pair_bias, mask) -> torch.Tensor:
         raise NotImplementedError("hip cross attention: gate / output projection biases")
     w = dict(q_w=module.linear_q.weight, q_b=module.linear_q.bias, k_w=module.linear_k.weight,
              v_w=module.linear_v.weight, g_w=module.linear_g.weight, o_w=module.linear_out.weight)
-    arith = select_arith(module, x_q)
+    arith = select_arith(module, x_q, call_site)
     C, H = module.channel_a, module.num_heads
     key = cache_key(tuple(w.values()), x_q, torch.float32 if arith == ops.KFH_ARITH_F32 else torch.bfloat16)
     blob = cached_blob(module, "_hip_cross_functional_cache", key,
@@ -146,8 +148,8 @@ def hip_attention_pair_bias(module: nn.Module, x_q: torch.Tensor, x_k: torch.Ten
     ``CrossAttentionPairBias`` (call site "diffusion_local")."""
     if x_q is not x_k and (x_q.shape != x_k.shape or x_q.data_ptr() != x_k.data_ptr()
                            or x_q.stride() != x_k.stride()):
-        return _run_cross(module, x_q, x_k, pair_bias, mask)
-    return _run(module, x_q, None, pair_bias, mask, apply_norm=False)
+        return _run_cross(module, x_q, x_k, pair_bias, mask, call_site)
+    return _run(module, x_q, None, pair_bias, mask, apply_norm=False, call_site=call_site)
 
 
 class AdaLN(nn.Module):
