@@ -81,8 +81,13 @@ int kfh_trimul_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w
                     const void* p_out_w, const void* g_out_w, int w_dtype, int C, void* blob,
                     void* stream);
 
-/* Workspace for one call with N tokens (per batch element; batches are processed in turn). */
+/* Workspace for one call with N tokens: enough for one batch element, batch elements are then
+ * processed in turn.  The *_batched size (>= the former) lets a call take all B elements through
+ * every kernel at once where the path supports it (the widths assembled from the token-track
+ * kernels, e.g. the C = 64 template stack, model/modules/apo_module.py:376-384 flattens templates
+ * into the batch); kfh_trimul_forward picks that mode when workspace_bytes suffices for it. */
 size_t kfh_trimul_workspace_bytes(int N, int C);
+size_t kfh_trimul_workspace_bytes_batched(int B, int N, int C);
 
 /* out[b,i,j,:] = (residual ? residual[b,i,j,:] : 0) + TriangleMultiplication(z, mask)[b,i,j,:]
  * z, out, residual: [B, N, N, C] contiguous, io_dtype.  mask: [B, N, N] bytes.
@@ -119,6 +124,9 @@ int kfh_triattn_pack(const void* ln_w, const void* ln_b, const void* q_w, const 
                      int w_dtype, int C, int H, void* blob, void* stream);
 
 size_t kfh_triattn_workspace_bytes(int N, int C, int H);
+/* as kfh_trimul_workspace_bytes_batched: all B elements through the projection kernels at once
+ * (the attention core stays one launch per element: its pair bias is the element's) */
+size_t kfh_triattn_workspace_bytes_batched(int B, int N, int C, int H);
 
 /* out = (residual or 0) + TriangleAttention{Starting,Ending}Node(x, mask).
  * x, out, residual: [B, N, N, C]; mask: [B, N, N] bytes (mask[b,i,k] gates key k of row i;

@@ -25,6 +25,7 @@ SIGNATURES: dict[str, tuple] = {
     "kfh_trimul_packed_bytes": (c_size_t, [c_int]),
     "kfh_trimul_pack": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, _P, _P]),
     "kfh_trimul_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "kfh_trimul_workspace_bytes_batched": (c_size_t, [c_int, c_int, c_int]),
     "kfh_trimul_forward": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                    c_float, c_int, _P]),
     "kfh_trimul_forward_stages": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
@@ -34,6 +35,7 @@ SIGNATURES: dict[str, tuple] = {
     "kfh_triattn_packed_bytes": (c_size_t, [c_int, c_int]),
     "kfh_triattn_pack": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_int, c_int, c_int, _P, _P]),
     "kfh_triattn_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "kfh_triattn_workspace_bytes_batched": (c_size_t, [c_int, c_int, c_int, c_int]),
     "kfh_triattn_forward": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                     c_int, c_float, c_int, _P]),
     "kfh_transition_packed_bytes": (c_size_t, [c_int, c_int]),

@@ -96,6 +96,12 @@ size_t kfh_trimul_workspace_bytes(int N, int C) {
     return planes_ab + planes_y;
 }
 
+size_t kfh_trimul_workspace_bytes_batched(int B, int N, int C) {
+    if (B <= 0) return 0;
+    if (trimul_generic(C)) return trimul_generic_ws_bytes(N, C, B);
+    return kfh_trimul_workspace_bytes(N, C);
+}
+
 int kfh_trimul_forward(const void* z, const uint8_t* mask, const void* blob, const void* residual,
                        void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                        int direction, float eps, int io_dtype, void* stream) {
@@ -125,12 +131,16 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
     const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
     char* ws = static_cast<char*>(workspace);
     if (trimul_generic(C)) {
-        for (int b = 0; b < B; ++b) {       // batch elements (templates) in turn through one workspace
+        // a workspace of kfh_trimul_workspace_bytes_batched(B, N, C) takes all batch elements
+        // (templates) through every kernel at once; a smaller one takes them in turn
+        const bool folded = B > 1 && workspace_bytes >= trimul_generic_ws_bytes(N, C, B);
+        const int step = folded ? B : 1;
+        for (int b = 0; b < B; b += step) {
             const size_t off = (size_t)b * N * N * C * esz;
             const int rc = trimul_generic_forward(
                 static_cast<const char*>(z) + off, io_dtype, mask + (size_t)b * N * N, static_cast<const char*>(blob),
-                ws, residual ? static_cast<const char*>(residual) + off : nullptr, static_cast<char*>(out) + off, N, C,
-                direction == KFH_INCOMING, eps, stages, stream);
+                ws, residual ? static_cast<const char*>(residual) + off : nullptr, static_cast<char*>(out) + off, step,
+                N, C, direction == KFH_INCOMING, eps, stages, stream);
             if (rc) return fail(KFH_EUNSUPPORTED, "trimul_forward: shape not built (%d)", rc);
         }
         return check_launch("trimul_forward");
@@ -229,6 +239,12 @@ size_t kfh_triattn_workspace_bytes(int N, int C, int H) {
     return ta_sizes(N).total;
 }
 
+size_t kfh_triattn_workspace_bytes_batched(int B, int N, int C, int H) {
+    if (B <= 0 || N <= 0 || N > 8192) return 0;
+    if (!triattn_fused(C, H)) return triattn_generic_ws_bytes(N, C, H, B);
+    return ta_sizes(N).total;
+}
+
 int kfh_triattn_forward(const void* x, const uint8_t* mask, const void* blob, const void* residual,
                         void* out, void* workspace, size_t workspace_bytes, int B, int N, int C,
                         int H, int ending, float eps, int io_dtype, void* stream) {
@@ -255,12 +271,16 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
         if (workspace_bytes < need)
             return fail(KFH_EINVAL, "triattn_forward: workspace %zu < %zu bytes", workspace_bytes, need);
         const size_t esz_g = io_dtype == KFH_F32 ? 4 : 2;
-        for (int b = 0; b < B; ++b) {       // batch elements (templates) in turn through one workspace
+        // a workspace of kfh_triattn_workspace_bytes_batched(B, N, C, H) takes all batch elements
+        // (templates) through the projection kernels at once; a smaller one takes them in turn
+        const bool folded = B > 1 && workspace_bytes >= triattn_generic_ws_bytes(N, C, H, B);
+        const int step = folded ? B : 1;
+        for (int b = 0; b < B; b += step) {
             const size_t off = (size_t)b * N * N * C * esz_g;
             const int rc = triattn_generic_forward(
                 static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N, static_cast<const char*>(blob),
                 static_cast<char*>(workspace), residual ? static_cast<const char*>(residual) + off : nullptr,
-                static_cast<char*>(out) + off, N, C, H, ending, eps, stages, stream);
+                static_cast<char*>(out) + off, step, N, C, H, ending, eps, stages, stream);
             if (rc) return fail(KFH_EUNSUPPORTED, "triattn_forward: shape not built (%d)", rc);
         }
         return check_launch("triattn_forward");

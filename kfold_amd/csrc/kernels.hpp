@@ -45,13 +45,14 @@ void launch_trimul_out(const uint16_t* planes_y, const void* z, const char* blob
 
 // any other width that is a multiple of 32 (trimul_generic.hip), from the token-track kernels
 size_t trimul_generic_blob_bytes(int C);
-size_t trimul_generic_ws_bytes(int N, int C);
+size_t trimul_generic_ws_bytes(int N, int C, int B = 1);
 int trimul_generic_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w, const void* g_in_w,
                         const void* ln_out_w, const void* ln_out_b, const void* p_out_w, const void* g_out_w,
                         int w_dtype, int C, void* blob, hipStream_t stream);
+// B batch elements at once (ws of trimul_generic_ws_bytes(N, C, B))
 int trimul_generic_forward(const void* z, int io_dtype, const uint8_t* mask, const char* blob, char* ws,
-                           const void* residual, void* out, int N, int C, int incoming, float eps, int stages,
-                           hipStream_t stream);
+                           const void* residual, void* out, int B, int N, int C, int incoming, float eps,
+                           int stages, hipStream_t stream);
 
 // other pair widths (trimul_wide.hip; C = 256): same interface, blob layout in that file
 size_t trimul_wide_blob_bytes(int C);
@@ -107,12 +108,14 @@ int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char*
 
 // other widths / head shapes (triattn_generic.hip): head dim <= 64, C a multiple of 32
 size_t triattn_generic_blob_bytes(int C, int H);
-size_t triattn_generic_ws_bytes(int N, int C, int H);
+size_t triattn_generic_ws_bytes(int N, int C, int H, int B = 1);
 int triattn_generic_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* k_w, const void* v_w,
                          const void* g_w, const void* bias_w, const void* o_w, int w_dtype, int C, int H,
                          void* blob, hipStream_t stream);
+// B batch elements at once (ws of triattn_generic_ws_bytes(N, C, H, B)); only the attention core is
+// launched per element
 int triattn_generic_forward(const void* x, int io_dtype, const uint8_t* mask, const char* blob, char* ws,
-                            const void* residual, void* out, int N, int C, int H, int ending, float eps,
+                            const void* residual, void* out, int B, int N, int C, int H, int ending, float eps,
                             int stages, hipStream_t stream);
 
 // ---- pair transition (transition.hip) ----------------------------------------------------
@@ -152,13 +155,16 @@ int launch_parcae_step(const void* z, const void* u, const void* u2, int io_dtyp
 int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const float* beta, uint16_t* out,
                      long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n = 0,
                      int parts = 1);
-// mask element of (row a, key k) is mask[a * mask_stride + k * key_stride]
+// mask element of (row a, key k) is mask[a * mask_stride + k * key_stride]; with rows_per_batch > 0
+// row a = b * rows_per_batch + i and the element is mask[b * batch_stride + i * mask_stride + k * key_stride]
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
-                      long long mask_stride, hipStream_t stream, long long key_stride = 1);
+                      long long mask_stride, hipStream_t stream, long long key_stride = 1,
+                      int rows_per_batch = 0, long long batch_stride = 0);
 // source element (t = batch*H + head, q, k) at t*st + q*sq + k*sk; all zero = dense [.., H, L, Lk];
-// L queries in nb blocks, Lk keys (0: = L)
+// with sb != 0 at batch*sb + head*st + q*sq + k*sk.  L queries in nb blocks, Lk keys (0: = L)
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
-                       hipStream_t stream, long long st = 0, long long sq = 0, long long sk = 0, int Lk = 0);
+                       hipStream_t stream, long long st = 0, long long sq = 0, long long sk = 0, int Lk = 0,
+                       long long sb = 0);
 // the same as fp32 tiles of 4 KiB (bias_tile_f32_elem layout) for the fp32 arithmetic
 void launch_bias_tiles_f32(const void* dense, int io_dtype, float* tiles, int nbatch, int H, int L, int nb,
                            hipStream_t stream, int Lk = 0);
@@ -179,6 +185,7 @@ struct LinearArgs {
     int epi;
     int H, PB, Dh;                               // heads, 32-blocks per padded head, real head dim
     int out_transposed;                          // EPI_RESID: out / aux row of (a, position) is position * rows_a + a
+                                                 // (inside each batch element of batch_rows row groups, see below)
     // fp32 arithmetic: parts = 3 — A, W, W2 and every bf16 output (row-major or fragments) are three
     // split3 planes, `*_part` bytes apart; the EPI_ADALN aux is summed over its three planes;
     // gate_dtype says how the EPI_RESID gate is stored (a KFH_F32 gate in this mode)
@@ -190,6 +197,11 @@ struct LinearArgs {
     // (a, position) is mask[a * L + position], or mask[position * rows_a + a] with mask_transposed.
     // EPI_RESID: optional mask byte per output row (0 zeroes the row)
     const uint8_t* mask; int mask_transposed;
+    // A batch folded into the row groups: a = b * batch_rows + i (batch_rows = 0: one element, i = a).
+    // Transposed indices (out_transposed, mask_transposed) are taken inside an element:
+    // b * batch_rows * L + position * batch_rows + i.  EPI_PLANES with nbatch > 1 stores channel c of
+    // element b at plane (c / plane_side) * nbatch * plane_side + b * plane_side + c % plane_side, row i.
+    int batch_rows, nbatch, plane_side;
 };
 int launch_linear(const LinearArgs& p, hipStream_t stream);
 

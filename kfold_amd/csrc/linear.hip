@@ -31,16 +31,21 @@ __device__ __forceinline__ void linear_epilogue(const LinearArgs& p, f32x16& acc
         // 32 lanes of a half write 32 consecutive positions of one plane
         const int ps = blk * 32 + col;
         if (ps >= p.L) return;
-        const size_t mi = p.mask_transposed ? (size_t)ps * p.rows_a + a : (size_t)a * p.L + ps;
+        const int br = p.batch_rows > 0 ? p.batch_rows : p.rows_a;      // row groups per batch element
+        const int bq = a / br, ai = a % br;
+        const size_t mi = p.mask_transposed ? ((size_t)bq * br * p.L + (size_t)ps * br + ai) : (size_t)a * p.L + ps;
         const bool valid = p.mask[mi] != 0;
         const size_t plane_sz = (size_t)p.ldo * p.ldo;
-        uint16_t* dst = static_cast<uint16_t*>(p.out) + (size_t)a * p.ldo + ps;
+        uint16_t* dst = static_cast<uint16_t*>(p.out) + (size_t)ai * p.ldo + ps;
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const int c = 32 * wb + acc_row(v, half);
             if (c >= p.Nout) continue;
+            const size_t plane = p.nbatch > 1 ? (size_t)(c / p.plane_side) * p.nbatch * p.plane_side +
+                                                    (size_t)bq * p.plane_side + c % p.plane_side
+                                              : (size_t)c;
             const float y = valid ? acc[v] * sigmoidf_fast(acc2[v]) : 0.f;
-            dst[(size_t)c * plane_sz] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
+            dst[plane * plane_sz] = (uint16_t)(pack_bf16(y, 0.f) & 0xffffu);
         }
     } else if constexpr (EPI == EPI_FRAG_CH || EPI == EPI_FRAG_POS) {
         const int h = wb / p.PB, pp = wb % p.PB;
@@ -91,7 +96,11 @@ __device__ __forceinline__ void linear_epilogue(const LinearArgs& p, f32x16& acc
             size_t r = (size_t)a * p.L + ps;
             size_t r_aux = (size_t)(p.aux_shared ? 0 : a) * p.L + ps;
             if constexpr (EPI == EPI_RESID) {
-                if (p.out_transposed) { r = (size_t)ps * p.rows_a + a; r_aux = r; }
+                if (p.out_transposed) {
+                    const int br = p.batch_rows > 0 ? p.batch_rows : p.rows_a;
+                    r = (size_t)(a / br) * br * p.L + (size_t)ps * br + a % br;
+                    r_aux = r;
+                }
             }
             const size_t r_gate = (size_t)(p.gate_shared ? 0 : a) * p.L + ps;
             float y = acc[v] + bc;

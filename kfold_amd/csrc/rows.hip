@@ -13,7 +13,8 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 // out[r', :] = bf16( normalize ? LN(x[r, :]) * gamma + beta : x[r, :] ), one wavefront per row.
 // gamma / beta may be null (1 / 0).  C is even, at most 2048.  With tn > 0 the rows are the
-// positions (i, j) of a [tn, tn] grid and are written transposed: r = i * tn + j -> r' = j * tn + i.
+// positions (i, j) of one or more [tn, tn] grids (a batch) and are written transposed inside their
+// grid: r = g * tn^2 + i * tn + j -> r' = g * tn^2 + j * tn + i.
 // (reference: model/primitives/normalization.py:61-91 — fp32 statistics, biased variance)
 // PARTS = 3: the fp32 result is written as its three split3 planes, plane q at out + q * M * C.
 template <int IO, int PARTS = 1>
@@ -25,7 +26,11 @@ __global__ __launch_bounds__(256) void rows_norm_kernel(const void* __restrict__
     const int lane = threadIdx.x & 63;
     const long long r = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (r >= M) return;
-    const long long ro = tn > 0 ? (r % tn) * tn + r / tn : r;
+    long long ro = r;
+    if (tn > 0) {
+        const long long grid = (long long)tn * tn, q = r % grid;
+        ro = r - q + (q % tn) * tn + q / tn;
+    }
     const int npair = (C + 127) / 128;
     float a[16], b[16];
     float s = 0.f;
@@ -84,7 +89,7 @@ int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const floa
                      long long M, int C, int normalize, float eps, hipStream_t stream, int transpose_n,
                      int parts) {
     if (C % 2 || C > 2048 || C <= 0) return -1;
-    if (transpose_n > 0 && (long long)transpose_n * transpose_n != M) return -1;
+    if (transpose_n > 0 && M % ((long long)transpose_n * transpose_n) != 0) return -1;
     if (parts != 1 && parts != 3) return -1;
     dim3 grid((unsigned)((M + 3) / 4)), block(256);
     if (parts == 3) {
@@ -105,30 +110,35 @@ int launch_rows_norm(const void* x, int io_dtype, const float* gamma, const floa
     return 0;
 }
 
-// codes[a][k] = k < L ? (mask[a * row_stride + k * key_stride] ? 2 : 1) : 0     for k < Lp = nb * 32
+// codes[a][k] = k < L ? (mask[b * batch_stride + i * row_stride + k * key_stride] ? 2 : 1) : 0  for k < Lp = nb * 32,
+// where row a = b * rows_per_batch + i (rows_per_batch = 0: one batch, i = a)
 __global__ void key_codes_kernel(const uint8_t* __restrict__ mask, uint8_t* __restrict__ codes,
-                                 int rows, int L, int Lp, long long row_stride, long long key_stride) {
+                                 int rows, int L, int Lp, long long row_stride, long long key_stride,
+                                 int rows_per_batch, long long batch_stride) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= (long long)rows * Lp) return;
     const int a = (int)(i / Lp), k = (int)(i % Lp);
-    codes[i] = k < L ? (mask[a * row_stride + k * key_stride] ? 2 : 1) : 0;
+    const int b = rows_per_batch > 0 ? a / rows_per_batch : 0, ai = rows_per_batch > 0 ? a % rows_per_batch : a;
+    codes[i] = k < L ? (mask[b * batch_stride + ai * row_stride + k * key_stride] ? 2 : 1) : 0;
 }
 
 void launch_key_codes(const uint8_t* mask, uint8_t* codes, int rows, int L, int Lp,
-                      long long mask_stride, hipStream_t stream, long long key_stride) {
+                      long long mask_stride, hipStream_t stream, long long key_stride, int rows_per_batch,
+                      long long batch_stride) {
     const long long n = (long long)rows * Lp;
     hipLaunchKernelGGL(key_codes_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, stream, mask,
-                       codes, rows, L, Lp, mask_stride, key_stride);
+                       codes, rows, L, Lp, mask_stride, key_stride, rows_per_batch, batch_stride);
 }
 
 // Dense pair bias [nbatch][H][L][L] -> log2(e)-scaled bf16 tiles (bias_tile_elem layout);
 // one thread writes the 8 keys of one (tile, chunk, lane) slot.
-// element (t, q, k) of the source is at t * st + q * sq + k * sk (t = batch * H + head); Lq x Lk
-// logits in nbq x nbk tiles
+// element (t, q, k) of the source is at t * st + q * sq + k * sk (t = batch * H + head), or with
+// hdiv > 0 at (t / hdiv) * sb + (t % hdiv) * st + q * sq + k * sk (a batch stride of its own);
+// Lq x Lk logits in nbq x nbk tiles
 template <int IO>
 __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __restrict__ tiles,
                                   long long total, int Lq, int Lk, int nbq, int nbk, long long st,
-                                  long long sq, long long sk) {
+                                  long long sq, long long sk, int hdiv, long long sb) {
     const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;      // 16-byte slot
     if (i >= total) return;
     const int lane = (int)(i & 63), c = (int)((i >> 6) & 1);
@@ -145,7 +155,8 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
             const int k = kb * 32 + acc_row(8 * c + e + u, lane >> 5);
             float x = 0.f;
             if (q < Lq && k < Lk) {
-                const size_t off = (size_t)(t * st + q * sq + k * sk);
+                const long long tb = hdiv > 0 ? (t / hdiv) * sb + (t % hdiv) * st : t * st;
+                const size_t off = (size_t)(tb + q * sq + k * sk);
                 if constexpr (IO == KFH_F32) x = static_cast<const float*>(dense)[off];
                 else x = bf16_lo(static_cast<const uint16_t*>(dense)[off]);
             }
@@ -157,7 +168,7 @@ __global__ void bias_tiles_kernel(const void* __restrict__ dense, uint16_t* __re
 }
 
 void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nbatch, int H, int L, int nb,
-                       hipStream_t stream, long long st, long long sq, long long sk, int Lk) {
+                       hipStream_t stream, long long st, long long sq, long long sk, int Lk, long long sb) {
     const int Lq = L, nbq = nb;
     if (Lk <= 0) Lk = L;
     const int nbk = (Lk + 31) / 32;
@@ -166,10 +177,10 @@ void launch_bias_tiles(const void* dense, int io_dtype, uint16_t* tiles, int nba
     dim3 grid((unsigned)((total + 255) / 256)), block(256);
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(bias_tiles_kernel<KFH_F32>, grid, block, 0, stream, dense, tiles, total, Lq, Lk, nbq,
-                           nbk, st, sq, sk);
+                           nbk, st, sq, sk, sb != 0 ? H : 0, sb);
     else
         hipLaunchKernelGGL(bias_tiles_kernel<KFH_BF16>, grid, block, 0, stream, dense, tiles, total, Lq, Lk, nbq,
-                           nbk, st, sq, sk);
+                           nbk, st, sq, sk, sb != 0 ? H : 0, sb);
 }
 
 // Dense pair bias -> log2(e)-scaled fp32 tiles (bias_tile_f32_elem layout): one thread writes the

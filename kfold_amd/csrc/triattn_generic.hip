@@ -39,27 +39,30 @@ struct TagLayout {
 };
 struct TagWs {
     size_t xn, qf, kf, vf, gf, of, bias, tiles, codes, total;
+    size_t frag1, tiles1, codes1;       // bytes of one batch element's fragments / bias tiles / key codes
     int nb;
-    TagWs(const TagLayout& l, int N) {
+    TagWs(const TagLayout& l, int N, int B) {
         nb = (N + 31) / 32;
         size_t off = 0;
         auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
-        xn = take((size_t)N * N * l.C * 2);
-        const size_t frag = (size_t)N * l.H * nb * l.PB * 2048;
-        qf = take(frag); kf = take(frag); vf = take(frag); gf = take(frag); of = take(frag);
-        bias = take((size_t)N * N * l.H * 2);
-        tiles = take((size_t)l.H * nb * nb * 2048);
-        codes = take((size_t)N * nb * 32);
+        xn = take((size_t)B * N * N * l.C * 2);
+        frag1 = (size_t)N * l.H * nb * l.PB * 2048;
+        qf = take(B * frag1); kf = take(B * frag1); vf = take(B * frag1); gf = take(B * frag1); of = take(B * frag1);
+        bias = take((size_t)B * N * N * l.H * 2);
+        tiles1 = (size_t)l.H * nb * nb * 2048;
+        tiles = take(B * tiles1);
+        codes1 = (size_t)N * nb * 32;
+        codes = take(B * codes1);
         total = off;
     }
 };
 }  // namespace
 
 size_t triattn_generic_blob_bytes(int C, int H) { return TagLayout(C, H).total; }
-size_t triattn_generic_ws_bytes(int N, int C, int H) {
+size_t triattn_generic_ws_bytes(int N, int C, int H, int B) {
     const TagLayout l(C, H);
-    if (!l.ok || N <= 0 || N > 8192) return 0;
-    return TagWs(l, N).total;
+    if (!l.ok || N <= 0 || N > 8192 || B <= 0) return 0;
+    return TagWs(l, N, B).total;
 }
 
 int triattn_generic_pack(const void* ln_w, const void* ln_b, const void* q_w, const void* k_w, const void* v_w,
@@ -89,20 +92,24 @@ int triattn_generic_pack(const void* ln_w, const void* ln_b, const void* q_w, co
     return 0;
 }
 
-// one batch element; returns 0 or a negative code of the failing launch helper
+// B batch elements: LayerNorm, projections, bias and the output projection run over the rows of all
+// elements at once (row group a = b * N + i); the attention core is launched per element (its
+// pair bias is the element's).  Returns 0 or a negative code of the failing launch helper.
 int triattn_generic_forward(const void* x, int io_dtype, const uint8_t* mask, const char* blob, char* ws,
-                            const void* residual, void* out, int N, int C, int H, int ending, float eps,
+                            const void* residual, void* out, int B, int N, int C, int H, int ending, float eps,
                             int stages, hipStream_t stream) {
     const TagLayout l(C, H);
-    if (!l.ok) return -1;
-    const TagWs w(l, N);
-    const long long rows = (long long)N * N;
+    if (!l.ok || B <= 0) return -1;
+    if ((long long)B * N > 0x7fffffffLL / 64) return -1;
+    const TagWs w(l, N, B);
+    const long long rows = (long long)B * N * N;
     uint16_t* xn = reinterpret_cast<uint16_t*>(ws + w.xn);
     const float* ln = reinterpret_cast<const float*>(blob + l.ln);
     auto base = [&](const void* A, long long lda, int K) {
         LinearArgs p{};
-        p.A = A; p.lda = lda; p.rows_a = N; p.L = N; p.nb = w.nb; p.K = K; p.bias_scale = 1.f;
+        p.A = A; p.lda = lda; p.rows_a = B * N; p.L = N; p.nb = w.nb; p.K = K; p.bias_scale = 1.f;
         p.H = H; p.PB = l.PB; p.Dh = l.Dh;
+        p.batch_rows = N; p.nbatch = B;
         return p;
     };
     if (stages & KFH_STAGE_IN) {
@@ -118,23 +125,28 @@ int triattn_generic_forward(const void* x, int io_dtype, const uint8_t* mask, co
         p.sigmoid = 0; p.epi = EPI_FRAG_POS;
         p.W = blob + l.wv; p.out = ws + w.vf;
         if (launch_linear(p, stream)) return -3;
-        // pair bias: [position (a, b)][head] -> tiles indexed (head, query a, key b)
+        // pair bias: [element][position (a, b)][head] -> tiles indexed (element, head, query a, key b)
+        if (rows > 0x7fffffffLL) return -3;
         LinearArgs pb{};
         pb.A = xn; pb.lda = C; pb.rows_a = 1; pb.L = (int)rows; pb.nb = (int)((rows + 31) / 32); pb.K = C;
         pb.W = blob + l.wb; pb.nblk = 1; pb.Nout = H; pb.bias_scale = 1.f; pb.H = 1; pb.PB = 1; pb.Dh = 32;
         pb.out = ws + w.bias; pb.out_dtype = KFH_BF16; pb.ldo = H; pb.epi = EPI_STORE;
         if (launch_linear(pb, stream)) return -3;
-        launch_bias_tiles(ws + w.bias, KFH_BF16, reinterpret_cast<uint16_t*>(ws + w.tiles), 1, H, N, w.nb, stream,
-                          1, (long long)N * H, H);
-        launch_key_codes(mask, reinterpret_cast<uint8_t*>(ws + w.codes), N, N, w.nb * 32, ending ? 1 : N, stream,
-                         ending ? N : 1);
+        launch_bias_tiles(ws + w.bias, KFH_BF16, reinterpret_cast<uint16_t*>(ws + w.tiles), B, H, N, w.nb, stream,
+                          1, (long long)N * H, H, 0, (long long)N * N * H);
+        launch_key_codes(mask, reinterpret_cast<uint8_t*>(ws + w.codes), B * N, N, w.nb * 32, ending ? 1 : N, stream,
+                         ending ? N : 1, N, (long long)N * N);
     }
     if (stages & KFH_STAGE_CORE) {
-        FlashArgs fa{};
-        fa.qf = ws + w.qf; fa.kf = ws + w.kf; fa.vf = ws + w.vf; fa.gf = ws + w.gf; fa.of = ws + w.of;
-        fa.biast = ws + w.tiles; fa.codes = reinterpret_cast<const uint8_t*>(ws + w.codes);
-        fa.nrows = N; fa.nb = w.nb; fa.H = H; fa.bias_per_row = 0;
-        if (launch_flash(fa, 32 * l.PB, stream)) return -4;
+        for (int b = 0; b < B; ++b) {
+            FlashArgs fa{};
+            fa.qf = ws + w.qf + b * w.frag1; fa.kf = ws + w.kf + b * w.frag1; fa.vf = ws + w.vf + b * w.frag1;
+            fa.gf = ws + w.gf + b * w.frag1; fa.of = ws + w.of + b * w.frag1;
+            fa.biast = ws + w.tiles + b * w.tiles1;
+            fa.codes = reinterpret_cast<const uint8_t*>(ws + w.codes + b * w.codes1);
+            fa.nrows = N; fa.nb = w.nb; fa.H = H; fa.bias_per_row = 0;
+            if (launch_flash(fa, 32 * l.PB, stream)) return -4;
+        }
     }
     if (stages & KFH_STAGE_OUT) {
         LinearArgs p = base(ws + w.of, 0, l.ko * 16);

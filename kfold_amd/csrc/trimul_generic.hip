@@ -40,31 +40,35 @@ struct TmgLayout {
 struct TmgWs {
     size_t xn, ab, y, yn, gate, total;
     int np;
-    TmgWs(const TmgLayout& l, int N) {
+    TmgWs(const TmgLayout& l, int N, int B) {
         np = trimul_np(N);
         size_t off = 0;
         auto take = [&](size_t bytes) { size_t o = off; off += align_up(bytes); return o; };
-        xn = take((size_t)N * N * l.C * 2);
-        ab = take((size_t)2 * l.C * np * np * 2);
-        y = take((size_t)l.C * np * np * 2);
-        yn = take((size_t)N * N * l.C * 2);
-        gate = take((size_t)N * N * l.C * 2);
+        xn = take((size_t)B * N * N * l.C * 2);
+        ab = take((size_t)B * 2 * l.C * np * np * 2);      // [a planes of all elements][b planes of all elements]
+        y = take((size_t)B * l.C * np * np * 2);
+        yn = take((size_t)B * N * N * l.C * 2);
+        gate = take((size_t)B * N * N * l.C * 2);
         total = off;
     }
 };
 
-// yn[row(i, j)][c] = LN_out over c of y[c][i][j] (fp32 statistics, biased variance), bf16; one
-// thread per position, three passes over its C plane values (the second and third hit L2).
+// yn[b][row(i, j)][c] = LN_out over c of y[b * C + c][i][j] (fp32 statistics, biased variance), bf16;
+// one thread per position, three passes over its C plane values (the second and third hit L2).
 // transposed: row(i, j) = j * N + i, else i * N + j.
 __global__ __launch_bounds__(256) void planes_norm_kernel(const uint16_t* __restrict__ planes,
                                                           const float* __restrict__ gamma,
                                                           const float* __restrict__ beta,
-                                                          uint16_t* __restrict__ out, int N, int Np, int C,
+                                                          uint16_t* __restrict__ out, int B, int N, int Np, int C,
                                                           float eps, int transposed) {
-    const long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= (long long)N * N) return;
+    long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= (long long)B * N * N) return;
+    const int b = (int)(idx / ((long long)N * N));
+    idx -= (long long)b * N * N;
     const int i = (int)(idx / N), j = (int)(idx % N);
     const size_t plane_sz = (size_t)Np * Np, pi = (size_t)i * Np + j;
+    planes += (size_t)b * C * plane_sz;
+    out += (size_t)b * N * N * C;
     float s = 0.f;
     for (int c = 0; c < C; ++c) s += bf16_lo(planes[c * plane_sz + pi]);
     const float mean = s / C;
@@ -84,10 +88,10 @@ __global__ __launch_bounds__(256) void planes_norm_kernel(const uint16_t* __rest
 }  // namespace
 
 size_t trimul_generic_blob_bytes(int C) { return TmgLayout(C).total; }
-size_t trimul_generic_ws_bytes(int N, int C) {
+size_t trimul_generic_ws_bytes(int N, int C, int B) {
     const TmgLayout l(C);
-    if (!l.ok || N <= 0) return 0;
-    return TmgWs(l, N).total;
+    if (!l.ok || N <= 0 || B <= 0) return 0;
+    return TmgWs(l, N, B).total;
 }
 
 int trimul_generic_pack(const void* ln_in_w, const void* ln_in_b, const void* p_in_w, const void* g_in_w,
@@ -108,15 +112,18 @@ int trimul_generic_pack(const void* ln_in_w, const void* ln_in_b, const void* p_
     return 0;
 }
 
-// one batch element; returns 0 or a negative code of the failing launch helper
+// B batch elements folded into the rows of every kernel (row group a = b * N + i); returns 0 or a
+// negative code of the failing launch helper
 int trimul_generic_forward(const void* z, int io_dtype, const uint8_t* mask, const char* blob, char* ws,
-                           const void* residual, void* out, int N, int C, int incoming, float eps, int stages,
-                           hipStream_t stream) {
+                           const void* residual, void* out, int B, int N, int C, int incoming, float eps,
+                           int stages, hipStream_t stream) {
     const TmgLayout l(C);
-    if (!l.ok) return -1;
-    const TmgWs w(l, N);
-    const long long rows = (long long)N * N;
+    if (!l.ok || B <= 0) return -1;
+    if ((long long)B * N > 0x7fffffffLL / 64) return -1;
+    const TmgWs w(l, N, B);
+    const long long rows = (long long)B * N * N;
     const int nb = (N + 31) / 32;
+    const size_t plane_sz = (size_t)w.np * w.np;
     uint16_t* xn = reinterpret_cast<uint16_t*>(ws + w.xn);
     uint16_t* ab = reinterpret_cast<uint16_t*>(ws + w.ab);
     uint16_t* y = reinterpret_cast<uint16_t*>(ws + w.y);
@@ -124,26 +131,27 @@ int trimul_generic_forward(const void* z, int io_dtype, const uint8_t* mask, con
     const float* ln = reinterpret_cast<const float*>(blob + l.ln);
     auto base = [&](const void* A, const void* W, int nout) {
         LinearArgs p{};
-        p.A = A; p.lda = C; p.rows_a = N; p.L = N; p.nb = nb; p.K = C; p.W = W; p.nblk = nout / 32; p.Nout = nout;
+        p.A = A; p.lda = C; p.rows_a = B * N; p.L = N; p.nb = nb; p.K = C; p.W = W; p.nblk = nout / 32; p.Nout = nout;
         p.bias_scale = 1.f; p.H = 1; p.PB = 1; p.Dh = 32;
+        p.batch_rows = N; p.nbatch = B; p.plane_side = C;
         return p;
     };
     if (stages & KFH_STAGE_IN) {
         // rows (a, pos): outgoing (i, k) = z[i, k]; incoming (i, k) = z[k, i] (written transposed)
         if (launch_rows_norm(z, io_dtype, ln, ln + C, xn, rows, C, 1, eps, stream, incoming ? N : 0)) return -2;
-        if (w.np != N) launch_fill_zero(ab, (size_t)2 * C * w.np * w.np * 2, stream);      // zero padding of the planes
+        if (w.np != N) launch_fill_zero(ab, (size_t)B * 2 * C * plane_sz * 2, stream);      // zero padding of the planes
         LinearArgs p = base(xn, blob + l.w_pin, 2 * C);
         p.W2 = blob + l.w_gin;
         p.epi = EPI_PLANES; p.out = ab; p.ldo = w.np;
         p.mask = mask; p.mask_transposed = incoming ? 1 : 0;
         if (launch_linear(p, stream)) return -3;
     }
-    if (stages & KFH_STAGE_CORE)
-        launch_contract(ab, ab + (size_t)C * w.np * w.np, y, w.np, C, stream);
+    if (stages & KFH_STAGE_CORE)      // one NT product per (element, channel): B * C planes on each side
+        launch_contract(ab, ab + (size_t)B * C * plane_sz, y, w.np, B * C, stream);
     if (stages & KFH_STAGE_OUT) {
         // transposed row order for the incoming direction: row (j, i) holds position (i, j)
         hipLaunchKernelGGL(planes_norm_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, stream, y,
-                           ln + 2 * C, ln + 3 * C, yn, N, w.np, C, eps, incoming ? 1 : 0);
+                           ln + 2 * C, ln + 3 * C, yn, B, N, w.np, C, eps, incoming ? 1 : 0);
         LinearArgs g = base(xn, blob + l.w_gout, C);
         g.epi = EPI_SIGMOID; g.out = ws + w.gate; g.out_dtype = KFH_BF16; g.ldo = C;
         if (launch_linear(g, stream)) return -3;

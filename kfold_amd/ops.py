@@ -71,15 +71,32 @@ def _workspace(given: torch.Tensor | None, need: int, dev: torch.device) -> torc
     return given
 
 
+# a batch is taken through the kernels at once when its workspace stays below this many bytes
+_BATCHED_WORKSPACE_CAP = 32 << 30
+
+
+def _batched_need(per_element: int, batched: int, given: torch.Tensor | None) -> int:
+    """Workspace size to ask for: the batched size if it is affordable (or the caller's buffer
+    already holds it), else the per-element size (batch elements then run in turn)."""
+    if batched > per_element and (batched <= _BATCHED_WORKSPACE_CAP if given is None else given.numel() >= batched):
+        return batched
+    return per_element
+
+
 def workspace_bytes(op: str, **shape) -> int:
     """Bytes of scratch memory a forward call needs (0: shape not supported): ``trimul`` (N, C),
-    ``triattn`` (N, C, heads), ``transition`` (rows, C, expansion), ``apb`` (S, L, C, heads,
+    ``triattn`` (N, C, heads) — both also with ``B``: the size that takes a batch through the kernels at
+    once —, ``transition`` (rows, C, expansion), ``apb`` (S, L, C, heads,
     cond_channels, arith), ``cross_apb`` (W, Lq, Lk, C, heads, cond_channels, arith).  Needs no GPU."""
     L = _lib.lib()
     g = shape.__getitem__
     if op == "trimul":
+        if "B" in shape:
+            return L.kfh_trimul_workspace_bytes_batched(g("B"), g("N"), g("C"))
         return L.kfh_trimul_workspace_bytes(g("N"), g("C"))
     if op == "triattn":
+        if "B" in shape:
+            return L.kfh_triattn_workspace_bytes_batched(g("B"), g("N"), g("C"), g("heads"))
         return L.kfh_triattn_workspace_bytes(g("N"), g("C"), g("heads"))
     if op == "transition":
         return L.kfh_transition_workspace_bytes(g("rows"), g("C"), g("expansion"))
@@ -145,6 +162,8 @@ def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, dire
     ws_bytes = L.kfh_trimul_workspace_bytes(N, C)
     if ws_bytes == 0:
         raise NotImplementedError(f"hip triangle multiplication takes C a multiple of 32 up to 256, got {C}")
+    if B > 1:
+        ws_bytes = _batched_need(ws_bytes, L.kfh_trimul_workspace_bytes_batched(B, N, C), workspace)
     ws = _workspace(workspace, ws_bytes, dev)
     d = KFH_INCOMING if direction == "incoming" else KFH_OUTGOING
     with torch.cuda.device(dev):
@@ -209,6 +228,8 @@ def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tens
     if ws_bytes == 0:
         raise NotImplementedError(
             f"hip triangle attention is built for C=128, H=4, N<=8192; got C={C}, H={heads}, N={N}")
+    if B > 1:
+        ws_bytes = _batched_need(ws_bytes, L.kfh_triattn_workspace_bytes_batched(B, N, C, heads), workspace)
     ws = _workspace(workspace, ws_bytes, dev)
     with torch.cuda.device(dev):
         check(L.kfh_triattn_forward(xc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),

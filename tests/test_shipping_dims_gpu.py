@@ -121,6 +121,44 @@ def test_triattn_other_widths_batched(starting, c, h, n, batch):
         assert_close(xin, x.float() + want, "residual in place", rel_fro=5e-3, auto_scale=True)
 
 
+@pytest.mark.parametrize("flip", [False, True])
+def test_template_batch_at_once_equals_templates_in_turn(flip):
+    """A workspace of the batched size takes all templates through the kernels at once, one of the
+    per-element size takes them in turn: same bits either way (c = 64, 4 templates)."""
+    from kfold_amd import ops, primitives as P
+
+    c, h, n, batch = 64, 4, 45, 4
+    print(f"case template batch folded vs in turn flip={flip}", flush=True)
+    g = torch.Generator().manual_seed(21)
+    x = torch.randn(batch, n, n, c, generator=g).bfloat16().to(DEV)
+    mask = (torch.rand(batch, n, n, generator=g) > 0.2).to(DEV)
+    tm = getattr(P, "TriangleMultiplicationIncoming" if flip else "TriangleMultiplicationOutgoing")(c).eval()
+    ta = getattr(P, "TriangleAttentionEndingNode" if flip else "TriangleAttentionStartingNode")(c, h).eval()
+    for m, seed in ((tm, 5), (ta, 6)):
+        synthetic.init_weights_(m, seed, std=0.08)
+        _affine(m)
+        m.to(DEV)
+    with torch.no_grad():
+        tm(x[:1], mask[:1]), ta(x[:1], mask[:1])       # packs the weights
+        one, many = ops.workspace_bytes("trimul", N=n, C=c), ops.workspace_bytes("trimul", N=n, C=c, B=batch)
+        assert many > one
+        direction = "incoming" if flip else "outgoing"
+        small = torch.empty(one + 256, dtype=torch.uint8, device=DEV)
+        small = small[(-small.data_ptr()) % 256:][:one]
+        a = ops.trimul_forward(x, mask, tm._hip_multiplication_cache, direction, workspace=small)
+        b = ops.trimul_forward(x, mask, tm._hip_multiplication_cache, direction)
+        assert torch.equal(a, b), "tri-mul: batch at once differs from elements in turn"
+        one, many = ops.workspace_bytes("triattn", N=n, C=c, heads=h), ops.workspace_bytes("triattn", N=n, C=c, heads=h, B=batch)
+        assert many > one
+        small = torch.empty(one + 256, dtype=torch.uint8, device=DEV)
+        small = small[(-small.data_ptr()) % 256:][:one]
+        a = ops.triattn_forward(x, mask, ta._hip_attention_cache, h, not flip, workspace=small)
+        b = ops.triattn_forward(x, mask, ta._hip_attention_cache, h, not flip)
+        assert torch.equal(a, b), "tri-attn: batch at once differs from elements in turn"
+        # the fused widths have no batched mode: same size either way
+        assert ops.workspace_bytes("trimul", N=n, C=128, B=batch) == ops.workspace_bytes("trimul", N=n, C=128)
+
+
 @pytest.mark.parametrize("direction", ["outgoing", "incoming"])
 @pytest.mark.parametrize("n", [384, 768])
 def test_trimul_c256_tiled_sizes(direction, n):
