@@ -29,7 +29,7 @@ CASES = [
     (TA, "test_triattn_long_sequence_sampled_rows", [()]),
     (TA, "test_triattn_config3_n512", [(True,), (False,)]),
     (SD, "test_triattn_c64_templates_n384", [(True,), (False,)]),
-    (SD, "test_trimul_c256_tiled_sizes", [(384, "outgoing"), (384, "incoming"), (768, "outgoing"), (768, "incoming")]),
+    (SD, "test_trimul_c256_tiled_sizes", [("outgoing", 384), ("incoming", 384), ("outgoing", 768), ("incoming", 768)]),
 ]
 
 

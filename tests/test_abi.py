@@ -37,6 +37,13 @@ def test_size_queries_and_argument_errors_need_no_gpu():
     # workspace grows with N and is 256-byte granular
     w1, w2 = lib.kfh_trimul_workspace_bytes(384, 128), lib.kfh_trimul_workspace_bytes(768, 128)
     assert 0 < w1 < w2 and w1 % 256 == 0
+    # batched sizes: the fused widths run batch elements in turn, the assembled ones can fold them
+    assert lib.kfh_trimul_workspace_bytes_batched(4, 384, 128) == w1
+    assert lib.kfh_trimul_workspace_bytes_batched(1, 100, 64) == lib.kfh_trimul_workspace_bytes(100, 64)
+    assert lib.kfh_trimul_workspace_bytes_batched(4, 100, 64) > 3 * lib.kfh_trimul_workspace_bytes(100, 64)
+    assert lib.kfh_triattn_workspace_bytes_batched(4, 100, 128, 4) == lib.kfh_triattn_workspace_bytes(100, 128, 4)
+    assert lib.kfh_triattn_workspace_bytes_batched(4, 100, 64, 4) > 3 * lib.kfh_triattn_workspace_bytes(100, 64, 4)
+    assert lib.kfh_trimul_workspace_bytes_batched(0, 100, 64) == 0 and lib.kfh_triattn_workspace_bytes_batched(4, 100, 48, 4) == 0
     assert lib.kfh_transition_workspace_bytes(1000, 128, 2) == 0       # fused pair kernel
     assert lib.kfh_transition_workspace_bytes(1000, 384, 4) > 0
     assert lib.kfh_apb_packed_bytes(384, 16, 0, 0) > 0 and lib.kfh_apb_packed_bytes(384, 5, 0, 0) == 0
