@@ -1,0 +1,63 @@
+"""bench.py's helpers that no GPU is needed for: the counter-summary reader, and the shipping-width
+rows of the configuration table run through the kernels' host build at small sizes (every module
+call of those rows executes; the times are stand-ins)."""
+
+import json
+import math
+
+import pytest
+
+
+def test_traffic_rows_follow_the_built_machine_code(tmp_path, monkeypatch):
+    import bench
+    from kfold_amd.build import ISA_JSON
+
+    if not ISA_JSON.exists():
+        pytest.skip("library not built by kfold_amd.build")
+    rows, why = bench.read_traffic_profile(768)
+    assert why is None, why
+    assert any(k.startswith("kfh::flash_strip_kernel") for k in rows)
+    for rd, wr in rows.values():
+        assert rd >= 0 and wr >= 0
+    # another N: no rows, with the reason
+    rows_n, why_n = bench.read_traffic_profile(512)
+    assert rows_n == {} and "N=768" in why_n
+    # a kernel whose machine code differs from the measured one loses its row
+    built = json.loads(ISA_JSON.read_text())
+    key = next(k for k in built if "flash_strip_kernel" in k)
+    built[key] = "0" * 16
+    other = tmp_path / "kernel_isa.json"
+    other.write_text(json.dumps(built))
+    import kfold_amd.build as kb
+
+    monkeypatch.setattr(kb, "ISA_JSON", other)
+    rows2, why2 = bench.read_traffic_profile(768)
+    assert why2 is None and not any(k.startswith("kfh::flash_strip_kernel") for k in rows2)
+    assert len(rows2) == len(rows) - 1
+    other.write_text("{}")
+    rows3, why3 = bench.read_traffic_profile(768)
+    assert rows3 == {} and "other machine code" in why3
+
+
+def test_shipping_width_rows_run_on_the_host_build():
+    import torch
+
+    import bench
+    from tests import hostsim
+
+    calls = []
+
+    def time_ms(fn):
+        fn()
+        calls.append(1)
+        return 1.0
+
+    with hostsim.host_backend(), torch.no_grad():
+        rows = bench.shipping_dim_rows(hostsim.HostDevice("cpu"), time_ms, n_wide=40, n_templates=36,
+                                       n_atoms_windows=2, n_tokens=40)
+    assert len(rows) == len(calls) == 7
+    assert [r["config"] for r in rows] == ["F2"] * 5 + ["F3"] * 2
+    for r in rows:
+        assert r["hip_ms"] == 1.0 and isinstance(r["what"], str) and isinstance(r["roof"], str)
+        assert r["tflops"] is None or (math.isfinite(r["tflops"]) and r["tflops"] > 0)
+    json.dumps(rows)
