@@ -49,19 +49,42 @@ ISA_FILES = ("trimul", "contract", "triattn", "flash", "transition", "pairbias")
 ISA_JSON = ROOT / "kernel_isa.json"
 
 
-def _isa_of(src: Path) -> dict[str, str]:
-    """{mangled kernel name: digest of its gfx950 instruction stream} for one source file.  Labels,
-    directives and comments are dropped, so the digest changes only when an instruction does."""
-    import hashlib
-    import re
+RESOURCES_JSON = ROOT / "kernel_resources.json"
+_RESOURCE_KEYS = ("vgpr_count", "agpr_count", "sgpr_count", "group_segment_fixed_size",
+                  "private_segment_fixed_size", "vgpr_spill_count", "max_flat_workgroup_size")
 
+
+def _asm_of(src: Path) -> str:
+    """gfx950 assembly (with the code object's metadata) of one source file."""
     res = subprocess.run([HIPCC, *FLAGS, "--cuda-device-only", "-S", str(src), "-o", "-"],
                          capture_output=True, text=True)
     if res.returncode != 0:
         raise RuntimeError(f"hipcc -S failed for {src.name}:\n{res.stderr[-2000:]}")
+    return res.stdout
+
+
+def _resources_of(asm: str) -> dict[str, dict[str, int]]:
+    """{mangled kernel name: registers, LDS bytes, scratch bytes per lane, spilled registers, largest
+    workgroup} as the compiler records them in the code object's metadata."""
+    import re
+
+    out = {}
+    for m in re.finditer(r"- \.agpr_count:.*?\.wavefront_size", asm, re.S):
+        block = m.group(0)
+        name = re.search(r"\.name:\s+(\S+)", block).group(1)
+        out[name] = {k: int(re.search(rf"\.{k}:\s+(\d+)", block).group(1)) for k in _RESOURCE_KEYS}
+    return out
+
+
+def _isa_of(asm: str) -> dict[str, str]:
+    """{mangled kernel name: digest of its gfx950 instruction stream} for one file's assembly.  Labels,
+    directives and comments are dropped, so the digest changes only when an instruction does."""
+    import hashlib
+    import re
+
     out: dict[str, list[str]] = {}
     cur = None
-    for line in res.stdout.splitlines():
+    for line in asm.splitlines():
         m = re.match(r"^(_Z\w+):", line)
         if m:
             cur = m.group(1)
@@ -81,12 +104,22 @@ def isa_digests(jobs: int = 8) -> dict[str, str]:
     """Digest of the compiled instruction stream of every kernel of the hot-path files: what a
     measurement (a rocprofv3 summary under profiles/) is valid for.  Edits that leave a kernel's
     machine code unchanged (comments, new helpers, other kernels) keep its digest."""
-    srcs = [CSRC / f"{name}.hip" for name in ISA_FILES]
-    merged: dict[str, str] = {}
+    return kernel_facts(jobs, [CSRC / f"{name}.hip" for name in ISA_FILES])[0]
+
+
+def kernel_facts(jobs: int = 8, srcs: list[Path] | None = None) -> tuple[dict[str, str], dict[str, dict[str, int]]]:
+    """(instruction-stream digests of the hot-path files' kernels, compiler-reported resources of
+    every kernel) from one assembly pass over the sources."""
+    srcs = sources() if srcs is None else srcs
+    hot = {CSRC / f"{name}.hip" for name in ISA_FILES}
+    isa: dict[str, str] = {}
+    res: dict[str, dict[str, int]] = {}
     with ThreadPoolExecutor(max_workers=jobs) as ex:
-        for d in ex.map(_isa_of, srcs):
-            merged.update(d)
-    return dict(sorted(merged.items()))
+        for src, asm in zip(srcs, ex.map(_asm_of, srcs)):
+            if src in hot:
+                isa.update(_isa_of(asm))
+            res.update(_resources_of(asm))
+    return dict(sorted(isa.items())), dict(sorted(res.items()))
 
 
 def build(verbose: bool = False, jobs: int | None = None) -> Path:
@@ -105,7 +138,9 @@ def build(verbose: bool = False, jobs: int | None = None) -> Path:
         raise RuntimeError(f"link failed:\n{res.stderr}")
     import json
 
-    ISA_JSON.write_text(json.dumps(isa_digests(), indent=1) + "\n")
+    isa, resources = kernel_facts(jobs)
+    ISA_JSON.write_text(json.dumps(isa, indent=1) + "\n")
+    RESOURCES_JSON.write_text(json.dumps(resources, indent=1) + "\n")
     return LIB
 
 

@@ -54,6 +54,8 @@ def load() -> ctypes.CDLL:
         h.hostsim_set_fill.argtypes = [c_int]
         h.hostsim_report.restype = None
         h.hostsim_report.argtypes = []
+        h.hostsim_launch_shapes.restype = c_size_t
+        h.hostsim_launch_shapes.argtypes = [ctypes.c_char_p, c_size_t]
         h.hostsim_threads.restype = c_int
         h.hostsim_threads.argtypes = []
         _sim = h

@@ -24,6 +24,11 @@ OBJ = HERE / "_obj"
 CXX = os.environ.get("HOSTSIM_CXX", "/opt/rocm/llvm/bin/clang++")
 FLAGS = ["-x", "c++", "-std=c++17", "-O2", "-march=x86-64-v3", "-fPIC", "-pthread", "-w",
          f"-I{HERE}", "-ffp-contract=off"]
+# extra compiler flags for a checking build, e.g.
+#   HOSTSIM_EXTRA_FLAGS="-fsanitize=alignment -fsanitize-trap=alignment" python tests/hostsim/build.py -f
+# makes every load and store through a typed pointer (the 16-byte fragment loads, the packed 4- and
+# 8-byte stores) trap unless the address has the type's alignment
+FLAGS += os.environ.get("HOSTSIM_EXTRA_FLAGS", "").split()
 
 
 def sources() -> list[Path]:

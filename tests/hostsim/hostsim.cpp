@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <thread>
+#include <string>
 #include <vector>
 
 namespace hostsim {
@@ -324,6 +325,9 @@ static void ensure_pool() {
 static std::mutex& g_launch_mu = *new std::mutex;
 static std::atomic<long long> g_launches{0};
 struct KernelStat { const char* name; long long launches, blocks; double seconds; };
+// largest workgroup each kernel was ever launched with (kept for the life of the process)
+struct KernelShape { const char* name; unsigned threads; };
+static std::vector<KernelShape>& g_shapes = *new std::vector<KernelShape>;
 static std::vector<KernelStat>& g_stats = *new std::vector<KernelStat>;
 static double now_s() {
     timespec ts;
@@ -334,6 +338,20 @@ static double now_s() {
 void launch(const char* name, dim3 grid, dim3 block, size_t dyn_lds, const std::function<void()>& body) {
     std::lock_guard<std::mutex> launch_lock(g_launch_mu);
     if (dyn_lds > 160 * 1024) die("dynamic LDS request above 160 KiB");
+    // what hipLaunchKernel refuses on the GPU
+    if (grid.y > 65535u || grid.z > 65535u || grid.x > 0x7fffffffu) die("grid dimension above the launch limit");
+    const unsigned long long nthreads = (unsigned long long)block.x * block.y * block.z;
+    if (nthreads == 0 || nthreads > (unsigned long long)kMaxThreadsPerBlock) die("workgroup size outside 1..1024");
+    {
+        bool seen = false;
+        for (KernelShape& k : g_shapes)
+            if (k.name == name || strcmp(k.name, name) == 0) {
+                if (k.threads < nthreads) k.threads = (unsigned)nthreads;
+                seen = true;
+                break;
+            }
+        if (!seen) g_shapes.push_back({name, (unsigned)nthreads});
+    }
     ensure_pool();
     g_launches++;
     Job j;
@@ -487,6 +505,19 @@ void hostsim_report(void) {
     hostsim::g_stats.clear();
 }
 long long hostsim_launch_count(void) { return hostsim::g_launches.load(); }
+// "name\tthreads\n" per kernel launched so far: the largest workgroup it was launched with;
+// returns the length needed (the text is cut to `cap` bytes including the final NUL)
+size_t hostsim_launch_shapes(char* buf, size_t cap) {
+    std::lock_guard<std::mutex> lk(hostsim::g_launch_mu);
+    std::string out;
+    for (const hostsim::KernelShape& k : hostsim::g_shapes) out += std::string(k.name) + "\t" + std::to_string(k.threads) + "\n";
+    if (buf && cap) {
+        const size_t n = out.size() < cap - 1 ? out.size() : cap - 1;
+        memcpy(buf, out.data(), n);
+        buf[n] = 0;
+    }
+    return out.size() + 1;
+}
 int hostsim_threads(void) { hostsim::ensure_pool(); return hostsim::g_threads; }
 
 }  // extern "C"
