@@ -50,6 +50,8 @@ def load() -> ctypes.CDLL:
         h.hostsim_launch_count.argtypes = []
         h.hostsim_set_schedule.restype = None
         h.hostsim_set_schedule.argtypes = [c_int]
+        h.hostsim_set_poison_lds.restype = None
+        h.hostsim_set_poison_lds.argtypes = [c_int]
         h.hostsim_set_fill.restype = None
         h.hostsim_set_fill.argtypes = [c_int]
         h.hostsim_report.restype = None

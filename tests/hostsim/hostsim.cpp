@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <thread>
+#include <link.h>
 #include <string>
 #include <vector>
 
@@ -97,6 +98,53 @@ char* dynamic_lds() { return t_worker->lds; }
 static std::atomic<int> g_skip_math{0};
 static std::atomic<int> g_schedule{0};      // order in which runnable lanes are resumed (see hostsim_set_schedule)
 static std::atomic<int> g_fill{1};
+static std::atomic<int> g_poison_lds{0};    // overwrite all LDS with 0xFF before every workgroup (see hostsim_set_poison_lds)
+
+// This thread's copy of the library's zero-initialised thread-local block: where every `__shared__`
+// array of the kernels lives in this build (one copy per worker thread, as a CU has one LDS).
+struct TlsSpan { char* base = nullptr; size_t bytes = 0; };
+static int find_tls(dl_phdr_info* info, size_t, void* out) {
+    const uintptr_t me = reinterpret_cast<uintptr_t>(&find_tls);
+    bool mine = false;
+    for (int i = 0; i < info->dlpi_phnum; ++i) {
+        const ElfW(Phdr)& ph = info->dlpi_phdr[i];
+        if (ph.p_type == PT_LOAD && me >= info->dlpi_addr + ph.p_vaddr && me < info->dlpi_addr + ph.p_vaddr + ph.p_memsz)
+            mine = true;
+    }
+    if (!mine) return 0;
+    for (int i = 0; i < info->dlpi_phnum; ++i) {
+        const ElfW(Phdr)& ph = info->dlpi_phdr[i];
+        if (ph.p_type == PT_TLS && info->dlpi_tls_data) {
+            TlsSpan* t = static_cast<TlsSpan*>(out);
+            t->base = static_cast<char*>(info->dlpi_tls_data) + ph.p_filesz;     // the part without initialisers
+            t->bytes = ph.p_memsz - ph.p_filesz;
+        }
+    }
+    return 1;
+}
+static void poison_lds(Worker* wk) {
+    static thread_local TlsSpan span;
+    static thread_local bool looked = false;
+    Worker* const w = t_worker;
+    Lane* const c = t_cur;
+    if (!looked) {
+        TlsSpan found;                  // a local: `span` itself lies in the block that is overwritten below
+        dl_iterate_phdr(find_tls, &found);
+        span = found;
+        looked = true;
+        if (getenv("HOSTSIM_DEBUG")) fprintf(stderr, "[hostsim] tls zero-init block %p + %zu (t_worker at %p)\n", (void*)found.base, found.bytes, (void*)&t_worker);
+    }
+    const TlsSpan keep = span;
+    if (keep.base) memset(keep.base, 0xFF, keep.bytes);
+    // the runtime's own thread-locals lie in the same block: let their addresses escape, so that the
+    // compiler takes the memset to have changed them and keeps the stores that put them back
+    asm volatile("" : : "r"(&t_worker), "r"(&t_cur), "r"(&span), "r"(&looked) : "memory");
+    span = keep;
+    looked = true;
+    t_worker = w;
+    t_cur = c;
+    memset(wk->lds, 0xFF, 160 * 1024);
+}
 
 [[noreturn]] static void die(const char* what) {
     Lane* c = t_cur;
@@ -181,6 +229,7 @@ static void run_block(Worker* wk, dim3 grid, dim3 block, dim3 bidx) {
     const int nt = (int)(block.x * block.y * block.z);
     if (nt > kMaxThreadsPerBlock || nt <= 0) die("workgroup size out of range");
     const int nw = (nt + 63) / 64;
+    if (g_poison_lds.load(std::memory_order_relaxed)) poison_lds(wk);
     wk->block = Block{};
     wk->block.alive = nt;
     for (int w = 0; w < nw; ++w) {
@@ -494,6 +543,10 @@ void hostsim_set_block_filter(long long stride, long long edge) {
 
 // 1 (default): new buffers are filled with 0xFF; 0: left as the zero pages the kernel maps
 void hostsim_set_fill(int on) { hostsim::g_fill.store(on); }
+// 1: every workgroup starts with all of its LDS (static arrays and the dynamic part) set to 0xFF
+// bytes, NaN as bf16 and as fp32, so a read of LDS that the workgroup has not written shows in the
+// result; costs a few MB of memset per workgroup, so it is for small problems
+void hostsim_set_poison_lds(int on) { hostsim::g_poison_lds.store(on); }
 // Order in which the lanes of a workgroup are resumed: 0 ascending, 1 descending, 2 wavefronts
 // rotating.  Results of a correctly synchronised kernel do not depend on it.
 void hostsim_set_schedule(int mode) { hostsim::g_schedule.store(mode); }

@@ -6,6 +6,10 @@ wavefront reads) gets whatever that order happens to produce.  Every kernel fami
 under three orders — lanes ascending, descending, wavefronts rotating from pass to pass — and has to
 give the same bits.  (A race between wavefronts that real hardware would expose shows here as a
 difference; lock-step effects inside one wavefront are outside what the model can vary.)
+
+A fourth run starts every workgroup with all of its LDS overwritten by 0xFF bytes (NaN as bf16 and
+fp32): a kernel that reads LDS it has not written itself (left over from the workgroup that ran on
+the compute unit before) gives other bits, or NaN.
 """
 
 from __future__ import annotations
@@ -19,14 +23,16 @@ from tests import hostsim
 
 def _run_all(build, run):
     outs = []
-    for mode in (0, 1, 2):
+    for mode, poison in ((0, 0), (1, 0), (2, 0), (0, 1)):
         mod = build()
         with torch.no_grad(), hostsim.host_backend():
             hostsim.load().hostsim_set_schedule(mode)
+            hostsim.load().hostsim_set_poison_lds(poison)
             try:
                 outs.append([t.clone() for t in run(mod)])
             finally:
                 hostsim.load().hostsim_set_schedule(0)
+                hostsim.load().hostsim_set_poison_lds(0)
     for other in outs[1:]:
         for a, b in zip(outs[0], other):
             assert torch.equal(a, b)
