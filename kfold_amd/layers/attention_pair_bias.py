@@ -75,6 +75,60 @@ def select_arith(module: nn.Module, x: torch.Tensor, call_site: str | None = Non
     return ops.KFH_ARITH_BF16
 
 
+class PairBiasTiles:
+    """A pair bias already in the attention kernel's tile order.
+
+    The diffusion sampler computes the pair bias of every transformer block once and uses it at
+    every step (model/modules/ecsi.py:506-512); converting the dense ``[*, H, L, L]`` tensor to tiles
+    on each call re-reads and re-writes it every time.  ``prepare_pair_bias`` does the conversion once;
+    the result is accepted wherever the self-attention entries take ``pair_bias``."""
+
+    def __init__(self, tiles: torch.Tensor, lead: tuple, heads: int, length: int, arith: int):
+        self.tiles, self.lead, self.heads, self.length, self.arith = tiles, tuple(lead), heads, length, arith
+
+    @property
+    def shape(self):
+        return self.lead + (self.heads, self.length, self.length)
+
+
+def prepare_pair_bias(pair_bias: torch.Tensor, arith: str | int = "bf16") -> PairBiasTiles:
+    """Dense pair bias ``[*, H, L, L]`` -> tiles for the arithmetic the attention will run in
+    ("bf16" or "f32": what ``select_arith`` gives for the call; a mismatch raises at the call)."""
+    if isinstance(arith, str):
+        if arith not in ("bf16", "f32"):
+            raise ValueError(f"arith must be 'bf16' or 'f32', got {arith!r}")
+        arith = ops.KFH_ARITH_F32 if arith == "f32" else ops.KFH_ARITH_BF16
+    if pair_bias.dim() < 3 or pair_bias.shape[-1] != pair_bias.shape[-2]:
+        raise ValueError(f"expected pair_bias [*, H, L, L], got {tuple(pair_bias.shape)}")
+    lead = tuple(pair_bias.shape[:-3])
+    flat = pair_bias.reshape((-1,) + pair_bias.shape[-3:])
+    return PairBiasTiles(ops.bias_tiles_from_dense(flat, arith), lead, pair_bias.shape[-3], pair_bias.shape[-1], arith)
+
+
+def _bias_tiles(pair_bias, lead: torch.Size, arith: int, heads: int, length: int):
+    """(tiles, one bias per flattened sample?) for a dense or a prepared pair bias."""
+    if isinstance(pair_bias, PairBiasTiles):
+        if pair_bias.arith != arith:
+            raise ValueError("the pair bias was prepared for the other arithmetic "
+                             f"({'f32' if pair_bias.arith == ops.KFH_ARITH_F32 else 'bf16'})")
+        if pair_bias.heads != heads or pair_bias.length != length:
+            raise ValueError(f"prepared pair bias {pair_bias.shape} does not match {heads} heads x {length} tokens")
+        n = 1
+        for d in pair_bias.lead:
+            n *= d
+        full = 1
+        for d in lead:
+            full *= d
+        if n == 1:
+            return pair_bias.tiles, False
+        if tuple(pair_bias.lead) != tuple(lead)[-len(pair_bias.lead):] or n != full:
+            raise ValueError(f"prepared pair bias {pair_bias.shape} must have one bias in all or the "
+                             f"leading dims {tuple(lead)} of the activations")
+        return pair_bias.tiles, True
+    pb, per_sample = _flatten(pair_bias, 3, lead)
+    return ops.bias_tiles_from_dense(pb, arith), per_sample
+
+
 def _flatten(t: torch.Tensor, keep: int, lead: torch.Size):
     """Flatten the leading dims of ``t`` (which broadcast against ``lead``) to 1 or prod(lead)."""
     tl = t.shape[:t.dim() - keep]
@@ -99,12 +153,11 @@ def _run(module, a, s, pair_bias, mask, apply_norm: bool, call_site: str | None 
     lead = a.shape[:-2]
     io = a if a.dtype in (torch.bfloat16, torch.float32) else a.float()
     af = io.reshape((-1,) + a.shape[-2:])
-    pb, per_sample = _flatten(pair_bias, 3, lead)
+    tiles, per_sample = _bias_tiles(pair_bias, lead, arith, H, a.shape[-2])
     mk, _ = _flatten(mask, 1, lead)
     sf = None
     if s is not None and apply_norm and Cs:
         sf, _ = _flatten(s, 2, lead)
-    tiles = ops.bias_tiles_from_dense(pb, arith)
     out = ops.apb_forward(af, sf, tiles, mk, blob, H, Cs, apply_norm, per_sample and af.shape[0] > 1,
                           eps=norm_eps(module), arith=arith)
     return out.reshape(a.shape).to(a.dtype)

@@ -294,3 +294,46 @@ def test_functional_entry_with_different_query_and_key_tensors(dtype):
                      rel_fro=1e-5)
     else:
         assert_close(got, want, "functional cross entry, bf16", auto_scale=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_prepared_pair_bias_gives_the_same_bits(dtype):
+    """The sampler computes each block's pair bias once and uses it at every step
+    (model/modules/ecsi.py:506-512): ``prepare_pair_bias`` converts it to tiles once; a call with the
+    prepared bias equals the call with the dense one bit for bit, in both arithmetics."""
+    from kfold_amd.layers import SelfAttentionPairBias, hip_attention_pair_bias, prepare_pair_bias
+
+    print(f"case prepared pair bias {dtype}", flush=True)
+    hip = SelfAttentionPairBias(768, 16, 384, "diffusion_global").eval()
+    synthetic.init_weights_(hip, 6, std=0.03)
+    hip.to(DEV)
+    L, S = 70, 3
+    g = torch.Generator().manual_seed(9)
+    a = torch.randn(1, S, L, 768, generator=g).to(dtype).to(DEV)
+    s = torch.randn(1, S, L, 384, generator=g).to(dtype).to(DEV)
+    bias = torch.randn(1, 1, 16, L, L, generator=g).to(DEV)
+    mask = (torch.rand(1, 1, L, generator=g) > 0.2).to(DEV)
+    arith = "f32" if dtype == torch.float32 else "bf16"
+    with torch.no_grad():
+        want = hip(a, s, bias, mask)
+        prepared = prepare_pair_bias(bias, arith)
+        assert prepared.shape == bias.shape
+        for _ in range(2):                                   # used again at the next step
+            assert torch.equal(hip(a, s, prepared, mask), want)
+        # one bias per sample
+        bias_s = torch.randn(1, S, 16, L, L, generator=g).to(DEV)
+        assert torch.equal(hip(a, s, prepare_pair_bias(bias_s, arith), mask), hip(a, s, bias_s, mask))
+        # the functional entry takes it as well
+        x = torch.randn(2, L, 768, generator=g).to(dtype).to(DEV)
+        b2 = torch.randn(2, 16, L, L, generator=g).to(DEV)
+        m2 = torch.ones(2, L, dtype=torch.bool).to(DEV)
+        site = "diffusion_global"
+        assert torch.equal(hip_attention_pair_bias(hip, x, x, prepare_pair_bias(b2, arith), m2, call_site=site),
+                           hip_attention_pair_bias(hip, x, x, b2, m2, call_site=site))
+        # prepared for the other arithmetic, or for another shape
+        with pytest.raises(ValueError):
+            hip(a, s, prepare_pair_bias(bias, "bf16" if arith == "f32" else "f32"), mask)
+        with pytest.raises(ValueError):
+            hip(a, s, prepare_pair_bias(bias[..., :L - 1, :L - 1].contiguous(), arith), mask)
+        with pytest.raises(ValueError):
+            hip(a, s, prepare_pair_bias(bias_s[:, :2].contiguous(), arith), mask)
