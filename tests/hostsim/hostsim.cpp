@@ -20,6 +20,7 @@
 #include <cstdlib>
 #include <mutex>
 #include <thread>
+#include <dlfcn.h>
 #include <link.h>
 #include <string>
 #include <vector>
@@ -488,6 +489,23 @@ static void segv_handler(int sig, siginfo_t* info, void*) {
     sigaction(sig, sig == SIGSEGV ? &g_old_segv : &g_old_bus, nullptr);
 }
 
+// A trap of a checking build (HOSTSIM_EXTRA_FLAGS with -fsanitize-trap): say where, as an offset
+// into this library that `llvm-symbolizer -e libkfold_hostsim.so` resolves when built with -g.
+static struct sigaction g_old_ill;
+static void ill_handler(int sig, siginfo_t* info, void*) {
+    Dl_info dl;
+    memset(&dl, 0, sizeof dl);
+    dladdr(info->si_addr, &dl);
+    fprintf(stderr, "\n[hostsim] trap at %p (library offset 0x%llx)", info->si_addr,
+            (unsigned long long)(static_cast<char*>(info->si_addr) - static_cast<char*>(dl.dli_fbase)));
+    if (t_worker) fprintf(stderr, " in kernel %s", t_worker->kernel);
+    if (t_cur)
+        fprintf(stderr, ", block (%u,%u,%u) thread %u", t_cur->bidx.x, t_cur->bidx.y, t_cur->bidx.z, t_cur->tidx.x);
+    fprintf(stderr, "\n");
+    fflush(stderr);
+    sigaction(sig, &g_old_ill, nullptr);
+}
+
 __attribute__((constructor)) static void install_handler() {
     // the handler runs on the faulting fiber's own stack, which is ordinary mapped memory
     struct sigaction sa;
@@ -496,6 +514,8 @@ __attribute__((constructor)) static void install_handler() {
     sa.sa_flags = SA_SIGINFO;
     sigaction(SIGSEGV, &sa, &g_old_segv);
     sigaction(SIGBUS, &sa, &g_old_bus);
+    sa.sa_sigaction = ill_handler;
+    sigaction(SIGILL, &sa, &g_old_ill);
 }
 
 }  // namespace hostsim
@@ -512,7 +532,7 @@ void* hostsim_alloc(size_t bytes, size_t align) {
     const size_t padded = (bytes + align - 1) / align * align;
     const size_t body = (padded + page - 1) / page * page;
     char* base = static_cast<char*>(mmap(nullptr, body + 2 * page, PROT_READ | PROT_WRITE,
-                                         MAP_PRIVATE | MAP_ANONYMOUS, -1, 0));
+                                         MAP_PRIVATE | MAP_ANONYMOUS | MAP_NORESERVE, -1, 0));
     if (base == MAP_FAILED) return nullptr;
     mprotect(base, page, PROT_NONE);
     mprotect(base + page + body, page, PROT_NONE);

@@ -174,3 +174,46 @@ def test_the_walk_has_teeth():
     assert "in-bounds call ok" in res.stdout
     assert "not reached" not in res.stdout and res.returncode != 0
     assert "[hostsim] invalid memory access" in res.stderr and "trimul_out_kernel" in res.stderr, res.stderr[-2000:]
+
+
+def _untouched(arena, shape, dtype):
+    """A guarded buffer that is never written (zero pages): at the sizes below the tensors are tens
+    of GB of address space of which only the sampled workgroups' pages are ever touched."""
+    n = 1
+    for d in shape:
+        n *= d
+    return arena.bytes(n * torch.empty((), dtype=dtype).element_size(), 256).view(dtype).view(shape)
+
+
+@pytest.mark.parametrize("what,n", [("pair_block", 3008), ("pair_block", 8192), ("wide_block", 6016),
+                                    ("template_block", 4000), ("diffusion_attention", 8192)])
+def test_walk_sizes_beyond_32_bit_offsets(what, n):
+    """Element offsets pass 2^31 from N = 2897 on at C = 128 (N^2 * 2C) and every entry point takes
+    N up to 8192: the first and last workgroups of every launch (and a stride between) at such sizes,
+    where an index computed in 32 bits would leave its buffer."""
+    from kfold_amd import layers, modules as M
+
+    hs = hostsim.load()
+    tok = synthetic.token_mask(n, synthetic.n_pad_for(n, 0.12))
+    with torch.no_grad(), _walk(stride=16411) as arena:
+        hs.hostsim_set_fill(0)
+        try:
+            if what == "pair_block":
+                blk = synthetic.init_weights_(M.PairSingleBlock().eval(), 0)
+                pm = synthetic.pair_mask_from_tokens(tok)
+                blk(_untouched(arena, (1, n, n, 128), torch.bfloat16), _untouched(arena, (1, n, 384), torch.bfloat16),
+                    arena.like(pm), arena.like(tok))
+            elif what == "wide_block":
+                blk = synthetic.init_weights_(M.TriangularBlock(256).eval(), 0)
+                blk(_untouched(arena, (1, n, n, 256), torch.bfloat16), arena.like(synthetic.pair_mask_from_tokens(tok)))
+            elif what == "template_block":
+                blk = synthetic.init_weights_(M.PairformerBlock(64, 4).eval(), 0)
+                pm = synthetic.pair_mask_from_tokens(tok).expand(2, n, n).contiguous()
+                blk(_untouched(arena, (2, n, n, 64), torch.bfloat16), arena.like(pm), inplace_output=True)
+            else:
+                for dtype in (torch.float32, torch.bfloat16):
+                    apb = synthetic.init_weights_(layers.SelfAttentionPairBias(768, 16, 384, "diffusion_global").eval(), 0)
+                    apb(_untouched(arena, (1, 5, n, 768), dtype), _untouched(arena, (1, 5, n, 384), dtype),
+                        _untouched(arena, (1, 1, 16, n, n), torch.float32), arena.like(tok.reshape(1, 1, n)))
+        finally:
+            hs.hostsim_set_fill(1)
