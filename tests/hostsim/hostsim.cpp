@@ -99,6 +99,7 @@ char* dynamic_lds() { return t_worker->lds; }
 static std::atomic<int> g_skip_math{0};
 static std::atomic<int> g_schedule{0};      // order in which runnable lanes are resumed (see hostsim_set_schedule)
 static std::atomic<int> g_fill{1};
+static std::atomic<int> g_strict_lanes{1};   // see wave_complete
 static std::atomic<int> g_poison_lds{0};    // overwrite all LDS with 0xFF before every workgroup (see hostsim_set_poison_lds)
 
 // This thread's copy of the library's zero-initialised thread-local block: where every `__shared__`
@@ -164,6 +165,12 @@ static void yield_to_scheduler() {
 }
 
 static void wave_complete(Wave* w) {
+    // Matrix and cross-lane data operations of a wavefront some of whose lanes have already left the
+    // kernel: the hardware takes the operands of such lanes from whatever their registers hold (MFMA
+    // does not look at the execution mask), so the result of the remaining lanes is not defined.
+    // Votes, readfirstlane and the wave barrier are defined for any set of active lanes.
+    if (w->alive != 64 && (w->tag == 1 || w->tag == 4 || w->tag == 6) && g_strict_lanes.load(std::memory_order_relaxed))
+        die("MFMA / shuffle / permlane in a wavefront with lanes that have exited");
     w->thunk(w->fnobj, w->slot, w->mask);
     for (int l = 0; l < 64; ++l) w->slot[l] = nullptr;
     w->mask = 0;
@@ -563,6 +570,7 @@ void hostsim_set_block_filter(long long stride, long long edge) {
 
 // 1 (default): new buffers are filled with 0xFF; 0: left as the zero pages the kernel maps
 void hostsim_set_fill(int on) { hostsim::g_fill.store(on); }
+void hostsim_set_strict_lanes(int on) { hostsim::g_strict_lanes.store(on); }
 // 1: every workgroup starts with all of its LDS (static arrays and the dynamic part) set to 0xFF
 // bytes, NaN as bf16 and as fp32, so a read of LDS that the workgroup has not written shows in the
 // result; costs a few MB of memset per workgroup, so it is for small problems
