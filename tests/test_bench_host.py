@@ -61,3 +61,14 @@ def test_shipping_width_rows_run_on_the_host_build():
         assert r["hip_ms"] == 1.0 and isinstance(r["what"], str) and isinstance(r["roof"], str)
         assert r["tflops"] is None or (math.isfinite(r["tflops"]) and r["tflops"] > 0)
     json.dumps(rows)
+
+
+def test_host_model_vectors_are_current():
+    """tests/golden/host_model_vectors.pt is what the host build gives today, bit for bit (a kernel
+    change that moves a result has to regenerate it: python -m tests.golden.make_host_model_vectors)."""
+    from tests import hostsim
+    from tests.test_zy_host_model_vectors_gpu import compare
+
+    with hostsim.host_backend():
+        stats = compare(hostsim.HostDevice("cpu"))
+    assert all(frac == 1.0 for frac, _ in stats.values()), stats
