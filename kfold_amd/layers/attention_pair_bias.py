@@ -143,6 +143,8 @@ def _run(module, a, s, pair_bias, mask, apply_norm: bool, call_site: str | None 
     check_inf(module)
     if module.linear_g.bias is not None or module.linear_out.bias is not None:
         raise NotImplementedError("hip pair-bias attention: gate / output projection biases")
+    if a.numel() == 0:                      # no samples or no tokens: nothing to attend to
+        return torch.empty_like(a)
     params = _parameters(module)
     C, H, Cs = module.channel_a, module.num_heads, _cond_channels(module)
     arith = select_arith(module, a, call_site)
@@ -171,6 +173,8 @@ def _run_cross(module, x_q, x_k, pair_bias, mask, call_site: str | None = None) 
     check_inf(module)
     if module.linear_g.bias is not None or module.linear_out.bias is not None:
         raise NotImplementedError("hip cross attention: gate / output projection biases")
+    if x_q.numel() == 0:                    # no windows or no queries
+        return torch.empty_like(x_q)
     w = dict(q_w=module.linear_q.weight, q_b=module.linear_q.bias, k_w=module.linear_k.weight,
              v_w=module.linear_v.weight, g_w=module.linear_g.weight, o_w=module.linear_out.weight)
     arith = select_arith(module, x_q, call_site)
@@ -321,6 +325,8 @@ class CrossAttentionPairBias(nn.Module):
             assert s_q is None and s_k is None
         if self.linear_g.bias is not None or self.linear_out.bias is not None:
             raise NotImplementedError("hip cross attention: gate / output projection biases")
+        if a_q.numel() == 0:                # no windows or no queries
+            return torch.empty_like(a_q)
         w = self._weights()
         cs = self.channel_s or 0
         arith = select_arith(self, a_q)

@@ -140,6 +140,10 @@ class PairSingleBlock(nn.Module):
         """``s += SelfAttentionPairBias(s; bias(z))``, ``s += Transition_4(s)`` on the current stream.
         ``after_bias`` is called once the last kernel that reads ``z`` has been enqueued."""
         B = z.shape[0]
+        if s.numel() == 0:                  # no tokens: nothing to update
+            if after_bias is not None:
+                after_bias()
+            return
         pb_params = (self.layernorm_z.weight, self.layernorm_z.bias, self.linear_pair_bias.weight)
         pb_blob = cached_blob(self, "_hip_pair_bias_cache", cache_key(pb_params, z, torch.bfloat16),
                               lambda: ops.pair_bias_pack(*pb_params, device=z.device))

@@ -203,3 +203,37 @@ def test_triangular_block():
             assert_close(zd, want, f"triangular block stage {i}", rel_fro=None)
         # the module call gives the same bits as the stage walk
         assert torch.equal(hip(zb.to(DEV), pmd), zd)
+
+
+def test_empty_inputs_give_empty_outputs():
+    """No tokens, no batch elements, no samples, no windows: every module returns an empty tensor
+    of the input's shape, as the reference's torch path does, without a kernel launch."""
+    from kfold_amd import layers, modules as M, primitives as P
+
+    print("case empty inputs", flush=True)
+    mk = lambda m: synthetic.init_weights_(m.eval(), 0).to(DEV)
+    z0 = torch.zeros(1, 0, 0, 128).bfloat16().to(DEV)
+    m0 = torch.zeros(1, 0, 0, dtype=torch.bool).to(DEV)
+    zb = torch.zeros(0, 8, 8, 128).bfloat16().to(DEV)
+    mb = torch.zeros(0, 8, 8, dtype=torch.bool).to(DEV)
+    f = lambda *shape: torch.zeros(*shape).to(DEV)
+    with torch.no_grad():
+        for mod in (mk(P.TriangleMultiplicationOutgoing(128)), mk(P.TriangleMultiplicationIncoming(128)),
+                    mk(P.TriangleAttentionStartingNode(128, 4)), mk(P.TriangleAttentionEndingNode(128, 4)),
+                    mk(P.TriangleMultiplicationOutgoing(64)), mk(P.TriangleAttentionStartingNode(64, 4))):
+            c = mod.linear_p_in.weight.shape[1] if hasattr(mod, "linear_p_in") else mod.c_in
+            assert mod(z0[..., :c], m0).shape == (1, 0, 0, c)
+            assert mod(zb[..., :c], mb).shape == (0, 8, 8, c)
+        assert mk(layers.Transition(128, 2))(f(0, 128)).shape == (0, 128)
+        assert mk(layers.Transition(384, 4))(f(0, 384)).shape == (0, 384)
+        apb = mk(layers.SelfAttentionPairBias(768, 16, 384, "diffusion_global"))
+        assert apb(f(1, 2, 0, 768), f(1, 2, 0, 384), f(1, 1, 16, 0, 0), m0.reshape(1, 1, 0)).shape == (1, 2, 0, 768)
+        assert apb(f(1, 0, 8, 768), f(1, 0, 8, 384), f(1, 1, 16, 8, 8),
+                   torch.ones(1, 1, 8, dtype=torch.bool).to(DEV)).shape == (1, 0, 8, 768)
+        cross = mk(layers.CrossAttentionPairBias(128, 4, 128))
+        assert cross(f(2, 0, 32, 128), f(2, 0, 128, 128), f(2, 0, 32, 128), f(2, 0, 128, 128), f(1, 0, 4, 32, 128),
+                     torch.ones(1, 0, 128, dtype=torch.bool).to(DEV)).shape == (2, 0, 32, 128)
+        assert M.ParcaeStep(128).eval().to(DEV)(f(1, 0, 0, 128), f(1, 0, 0, 128)).shape == (1, 0, 0, 128)
+        zz, ss = mk(M.PairSingleBlock())(z0, torch.zeros(1, 0, 384).bfloat16().to(DEV), m0,
+                                        torch.zeros(1, 0, dtype=torch.bool).to(DEV))
+        assert zz.shape == (1, 0, 0, 128) and ss.shape == (1, 0, 384)
