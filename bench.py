@@ -529,6 +529,9 @@ def main() -> int:
     ap.add_argument("--no-extras", action="store_true",
                     help="skip the per-kernel table, the unpadded / large-logit timings and the 48-block trunk")
     ap.add_argument("--table", action="store_true", help="also measure every benchmark configuration")
+    ap.add_argument("--phase-chunks", type=int, default=0,
+                    help="also time the block with every triangle op's core and output phase overlapped over this "
+                         "many ranges of rows (same results bit for bit; reported beside the headline, never as it)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); "
@@ -580,6 +583,19 @@ def main() -> int:
             torch.cuda.synchronize()
             timings[name] = (time.perf_counter() - t0) * 1e3 / args.steps
         ms_per_step = timings["overlapped"]
+        if args.phase_chunks > 1:
+            block.pair_block.phase_row_chunks = args.phase_chunks
+            try:
+                for name, overlap in (("phases_serial_tracks", False), ("phases_overlapped_tracks", True)):
+                    z, s = h.z0.clone(), h.s0.clone()
+                    chain(args.warmup, z, s, overlap)
+                    torch.cuda.synchronize()
+                    t0 = time.perf_counter()
+                    chain(args.steps, z, s, overlap)
+                    torch.cuda.synchronize()
+                    timings[name] = (time.perf_counter() - t0) * 1e3 / args.steps
+            finally:
+                block.pair_block.phase_row_chunks = 1
 
         # ---- per-op times (fresh inputs so the values are those of the first block) ---------
         zb, sb = h.z0, h.s0.clone()
@@ -650,6 +666,10 @@ def main() -> int:
                                "pair track of step k+1 (serial_schedule_ms_per_step: everything on one stream)"},
         "schedule": "single track of step k on a second stream beside the pair track of step k+1",
         "serial_schedule_ms_per_step": round(timings["serial"], 4),
+        **({"phase_overlap": {"row_chunks": args.phase_chunks,
+                              "ms_per_step_tracks_serial": round(timings["phases_serial_tracks"], 4),
+                              "ms_per_step_tracks_overlapped": round(timings["phases_overlapped_tracks"], 4)}}
+           if "phases_serial_tracks" in timings else {}),
         "block_tflops": round(fl["block"] / ms_per_step / 1e9, 1),
         "block_mfma_frac": round(fl["block"] / ms_per_step / 1e9 / PEAK_BF16_TFLOPS, 4),
         "ops": ops_ms,

@@ -108,6 +108,21 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
                               const void* residual, void* out, void* workspace,
                               size_t workspace_bytes, int B, int N, int C, int direction, float eps,
                               int io_dtype, int stages, void* stream);
+/* The stages over a range of result rows: KFH_STAGE_CORE and KFH_STAGE_OUT take rows
+ * [row0, row0 + nrows) of the result (out[b, i, :, :] for i in the range, both directions);
+ * KFH_STAGE_IN always makes all rows and is called once, with row0 = 0, nrows = N.  For a caller
+ * that overlaps the phases of one op: the contraction of one range on one stream beside the output
+ * phase (LayerNorm, gate, projection, residual: memory-bound) of the range before on another,
+ * ordered by the caller's events (the reference has no counterpart: its op is one call,
+ * model/primitives/triangle_multiplication.py:212-229).  The ranges run the kernels of the whole op
+ * on offset pointers: results have the bits of kfh_trimul_forward.  B = 1, C = 128 or 256; row0 a
+ * multiple of kfh_trimul_row_granule(N, C) (the contraction's tile rows), nrows as well unless the
+ * range ends at N. */
+int kfh_trimul_row_granule(int N, int C);
+int kfh_trimul_forward_rows(const void* z, const uint8_t* mask, const void* blob,
+                            const void* residual, void* out, void* workspace,
+                            size_t workspace_bytes, int B, int N, int C, int direction, float eps,
+                            int io_dtype, int stages, int row0, int nrows, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Triangle attention around the starting / ending node (Algorithms 14/15).
@@ -146,6 +161,15 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
                                const void* residual, void* out, void* workspace,
                                size_t workspace_bytes, int B, int N, int C, int H, int ending,
                                float eps, int io_dtype, int stages, void* stream);
+/* As kfh_trimul_forward_rows: attention (KFH_STAGE_CORE) and output phase (KFH_STAGE_OUT) over the
+ * attention rows [row0, row0 + nrows) — x[b, i] for the starting node, x[b, :, i] for the ending node
+ * (model/primitives/triangle_attention.py:400-402) —, KFH_STAGE_IN over all rows.  B = 1, C = 128,
+ * H = 4; a range has 48 rows at least when N >= 48 (the attention kernel of the whole op must take
+ * the range as well, so that the bits are those of kfh_triattn_forward). */
+int kfh_triattn_forward_rows(const void* x, const uint8_t* mask, const void* blob,
+                             const void* residual, void* out, void* workspace,
+                             size_t workspace_bytes, int B, int N, int C, int H, int ending,
+                             float eps, int io_dtype, int stages, int row0, int nrows, void* stream);
 
 /* ---------------------------------------------------------------------------------------
  * Transition (Algorithm 11, SwiGLU).  Replaces the torch modules

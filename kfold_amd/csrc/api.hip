@@ -113,6 +113,19 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
                               const void* residual, void* out, void* workspace,
                               size_t workspace_bytes, int B, int N, int C, int direction, float eps,
                               int io_dtype, int stages, void* stream_) {
+    return kfh_trimul_forward_rows(z, mask, blob, residual, out, workspace, workspace_bytes, B, N, C, direction,
+                                   eps, io_dtype, stages, 0, N, stream_);
+}
+
+int kfh_trimul_row_granule(int N, int C) {
+    if ((C != kC && !trimul_wide(C)) || N <= 0) return 0;
+    return contract_tile_rows(trimul_np(N));
+}
+
+int kfh_trimul_forward_rows(const void* z, const uint8_t* mask, const void* blob,
+                            const void* residual, void* out, void* workspace,
+                            size_t workspace_bytes, int B, int N, int C, int direction, float eps,
+                            int io_dtype, int stages, int row0, int nrows, void* stream_) {
     if (C != kC && !trimul_wide(C) && !trimul_generic(C))
         return fail(KFH_EUNSUPPORTED, "trimul_forward: C=%d (a multiple of 32 up to 256)", C);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "trimul_forward: bad shape B=%d N=%d", B, N);
@@ -123,6 +136,15 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
         return fail(KFH_EINVAL, "trimul_forward: null pointer argument");
     if (out == z && residual != z)
         return fail(KFH_EINVAL, "trimul_forward: out may alias z only when residual == z");
+    const bool ranged = row0 != 0 || nrows != N;
+    if (ranged) {
+        const int granule = kfh_trimul_row_granule(N, C);
+        if (granule == 0 || B != 1)
+            return fail(KFH_EUNSUPPORTED, "trimul_forward_rows: row ranges take B = 1 and C = 128 or 256 (B=%d C=%d)", B, C);
+        if (row0 < 0 || nrows < 0 || row0 + nrows > N || row0 % granule || (nrows % granule && row0 + nrows != N))
+            return fail(KFH_EINVAL, "trimul_forward_rows: rows [%d, %d) of %d (ranges start at multiples of %d)", row0,
+                        row0 + nrows, N, granule);
+    }
     const size_t need = kfh_trimul_workspace_bytes(N, C);
     if (workspace_bytes < need)
         return fail(KFH_EINVAL, "trimul_forward: workspace %zu < %zu bytes", workspace_bytes, need);
@@ -161,13 +183,16 @@ int kfh_trimul_forward_stages(const void* z, const uint8_t* mask, const void* bl
                 launch_trimul_in(zb, io_dtype, mask + (size_t)b * N * N, bl, planes_ab, N, np,
                                  direction == KFH_INCOMING, eps, stream);
         }
+        // the input phase always makes all rows of the planes; the last range of the contraction
+        // also takes the padded rows below N
+        const int crows = row0 + nrows == N ? np - row0 : nrows;
         if (stages & KFH_STAGE_CORE)
-            launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream);
+            launch_contract(planes_ab, planes_ab + (size_t)C * np * np, planes_y, np, C, stream, row0, crows);
         if (stages & KFH_STAGE_OUT) {
             if (trimul_wide(C))
-                launch_trimul_out_wide(planes_y, zb, bl, rb, ob, io_dtype, N, np, C, eps, stream);
+                launch_trimul_out_wide(planes_y, zb, bl, rb, ob, io_dtype, N, np, C, eps, stream, row0, nrows);
             else
-                launch_trimul_out(planes_y, zb, bl, rb, ob, io_dtype, N, np, eps, stream);
+                launch_trimul_out(planes_y, zb, bl, rb, ob, io_dtype, N, np, eps, stream, row0, nrows);
         }
     }
     return check_launch("trimul_forward");
@@ -256,6 +281,14 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
                                const void* residual, void* out, void* workspace,
                                size_t workspace_bytes, int B, int N, int C, int H, int ending,
                                float eps, int io_dtype, int stages, void* stream_) {
+    return kfh_triattn_forward_rows(x, mask, blob, residual, out, workspace, workspace_bytes, B, N, C, H, ending,
+                                    eps, io_dtype, stages, 0, N, stream_);
+}
+
+int kfh_triattn_forward_rows(const void* x, const uint8_t* mask, const void* blob,
+                             const void* residual, void* out, void* workspace,
+                             size_t workspace_bytes, int B, int N, int C, int H, int ending,
+                             float eps, int io_dtype, int stages, int row0, int nrows, void* stream_) {
     if (!triattn_fused(C, H) && triattn_generic_blob_bytes(C, H) == 0)
         return fail(KFH_EUNSUPPORTED, "triattn_forward: C=%d H=%d (C a multiple of 32, head dim <= 64)", C, H);
     if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "triattn_forward: bad shape B=%d N=%d", B, N);
@@ -265,6 +298,12 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
         return fail(KFH_EINVAL, "triattn_forward: null pointer argument");
     if (out == x && residual != x)
         return fail(KFH_EINVAL, "triattn_forward: out may alias x only when residual == x");
+    if (row0 != 0 || nrows != N) {
+        if (!triattn_fused(C, H) || B != 1)
+            return fail(KFH_EUNSUPPORTED, "triattn_forward_rows: row ranges take B = 1, C = 128, H = 4 (B=%d C=%d H=%d)", B, C, H);
+        if (row0 < 0 || nrows < 0 || row0 + nrows > N)
+            return fail(KFH_EINVAL, "triattn_forward_rows: rows [%d, %d) of %d", row0, row0 + nrows, N);
+    }
     hipStream_t stream = static_cast<hipStream_t>(stream_);
     if (!triattn_fused(C, H)) {
         const size_t need = triattn_generic_ws_bytes(N, C, H);
@@ -305,7 +344,10 @@ int kfh_triattn_forward_stages(const void* x, const uint8_t* mask, const void* b
         const int rc = launch_triattn(static_cast<const char*>(x) + off, io_dtype, mask + (size_t)b * N * N,
                                       static_cast<const char*>(blob), ws,
                                       residual ? static_cast<const char*>(residual) + off : nullptr,
-                                      static_cast<char*>(out) + off, N, ending, eps, stages, stream);
+                                      static_cast<char*>(out) + off, N, ending, eps, stages, stream, row0, nrows);
+        if (rc == -3)
+            return fail(KFH_EINVAL, "triattn_forward_rows: a range of %d rows is too short for the attention kernel of "
+                        "N = %d (48 rows at least)", nrows, N);
         if (rc) return fail(KFH_EHIP, "triattn_forward: attention kernel launch failed (%d)", rc);
     }
     return check_launch("triattn_forward");

@@ -187,19 +187,25 @@ __global__ __launch_bounds__(256, OCC) void contract_kernel(const uint16_t* __re
 }
 
 void launch_contract(const uint16_t* planes_a, const uint16_t* planes_b, uint16_t* planes_y,
-                     int Np, int D, hipStream_t stream) {
+                     int Np, int D, hipStream_t stream, int row0, int nrows) {
     // Np is a multiple of 128; use 256x256 tiles when they divide it, else 128x128.
     // (192x256 tiles fill the CUs evenly at Np = 768, 6 rounds instead of 4.5, but measured
     // slower: 189 against 161-177 us.)
-    if (Np % 256 == 0) {
-        const int t = Np / 256;
-        hipLaunchKernelGGL((contract_kernel<4, 4, 64, 1>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
-                           planes_b, planes_y, Np, t, t);
-    } else {
-        const int t = Np / 128;
-        hipLaunchKernelGGL((contract_kernel<2, 2, 64, 2>), dim3(D * t * t), dim3(256), 0, stream, planes_a,
-                           planes_b, planes_y, Np, t, t);
-    }
+    // a range of result rows = the tile rows that hold it: the A and Y planes are entered row0 rows
+    // down (the plane stride stays Np * Np), B is used whole
+    const int bm = contract_tile_rows(Np);
+    if (nrows < 0) { row0 = 0; nrows = Np; }
+    const int tm0 = row0 / bm, tm1 = (row0 + nrows + bm - 1) / bm;
+    if (tm1 <= tm0) return;
+    planes_a += (size_t)tm0 * bm * Np;
+    planes_y += (size_t)tm0 * bm * Np;
+    const int tn = Np / bm;
+    if (bm == 256)
+        hipLaunchKernelGGL((contract_kernel<4, 4, 64, 1>), dim3(D * (tm1 - tm0) * tn), dim3(256), 0, stream, planes_a,
+                           planes_b, planes_y, Np, tm1 - tm0, tn);
+    else
+        hipLaunchKernelGGL((contract_kernel<2, 2, 64, 2>), dim3(D * (tm1 - tm0) * tn), dim3(256), 0, stream, planes_a,
+                           planes_b, planes_y, Np, tm1 - tm0, tn);
 }
 
 }  // namespace kfh

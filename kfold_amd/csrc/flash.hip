@@ -694,13 +694,18 @@ static int launch_strip(FlashArgs p, hipStream_t stream) {
     return 0;
 }
 
-int launch_flash(const FlashArgs& args_in, int head_dim_pad, hipStream_t stream) {
+int launch_flash(const FlashArgs& args_in, int head_dim_pad, hipStream_t stream, int full_rows) {
     FlashArgs args = args_in;
     if (args.nbq <= 0) args.nbq = args.nb;            // self attention
     if (args.nb > 256 || args.nbq > 256) return -1;
-    if (!args.bias_per_row && args.nbq == args.nb && head_dim_pad == 32 && args.nb <= kStripMaxBlocks &&
-        args.nrows >= 4 * kStripWaves)
+    const bool strip_shape = !args.bias_per_row && args.nbq == args.nb && head_dim_pad == 32 &&
+                             args.nb <= kStripMaxBlocks;
+    if (strip_shape && (full_rows > 0 ? full_rows : args.nrows) >= 4 * kStripWaves) {
+        // a range of rows runs on the kernel the whole problem runs on (the two kernels visit the
+        // key blocks in different orders and do not give the same bits)
+        if (args.nrows < 4 * kStripWaves) return -3;
         return launch_strip(args, stream);
+    }
     return launch_staged(args, head_dim_pad, stream);
 }
 

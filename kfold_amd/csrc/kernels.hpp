@@ -37,11 +37,16 @@ inline int trimul_np(int N) { return round_up(N, 128); }
 
 void launch_trimul_in(const void* z, int io_dtype, const uint8_t* mask, const char* blob,
                       uint16_t* planes, int N, int Np, int incoming, float eps, hipStream_t stream);
+// rows of one contraction tile at this plane size: a range of result rows handed to
+// launch_contract starts at a multiple of it
+inline int contract_tile_rows(int Np) { return Np % 256 == 0 ? 256 : 128; }
+// row0 / nrows: only the result rows [row0, row0 + nrows) of every plane (nrows < 0: all Np rows);
+// the same kernels on offset pointers, so a result computed in ranges has the bits of one launch
 void launch_contract(const uint16_t* planes_a, const uint16_t* planes_b, uint16_t* planes_y,
-                     int Np, int D, hipStream_t stream);
+                     int Np, int D, hipStream_t stream, int row0 = 0, int nrows = -1);
 void launch_trimul_out(const uint16_t* planes_y, const void* z, const char* blob,
                        const void* residual, void* out, int io_dtype, int N, int Np, float eps,
-                       hipStream_t stream);
+                       hipStream_t stream, int row0 = 0, int nrows = -1);
 
 // any other width that is a multiple of 32 (trimul_generic.hip), from the token-track kernels
 size_t trimul_generic_blob_bytes(int C);
@@ -60,7 +65,8 @@ void trimul_wide_offsets(int C, size_t* gate, size_t* ab, size_t* out, size_t* l
 int launch_trimul_in_wide(const void* z, int io_dtype, const uint8_t* mask, const char* blob, uint16_t* planes,
                           int N, int Np, int C, int incoming, float eps, hipStream_t stream);
 int launch_trimul_out_wide(const uint16_t* planes_y, const void* z, const char* blob, const void* residual,
-                           void* out, int io_dtype, int N, int Np, int C, float eps, hipStream_t stream);
+                           void* out, int io_dtype, int N, int Np, int C, float eps, hipStream_t stream,
+                           int row0 = 0, int nrows = -1);
 
 // ---- triangle attention (triattn.hip) ------------------------------------------------------
 // Packed weight blob of one triangle-attention module (C = 128, 4 heads x 32):
@@ -96,7 +102,9 @@ struct FlashArgs {
     // (split3), `*_part` bytes apart; the bias tiles are fp32 (bias_tile_f32_elem layout)
     size_t q_part, k_part, v_part, g_part, o_part;
 };
-int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
+// full_rows > 0: args describe a range of the rows of a problem with full_rows rows; the kernel is
+// chosen as for the whole problem (returns -3 if the range is too short for that kernel)
+int launch_flash(const FlashArgs& args, int head_dim_pad, hipStream_t stream, int full_rows = 0);
 // the same attention in fp32 arithmetic on split operands (flash_split.hip)
 int launch_flash_split(const FlashArgs& args, int head_dim_pad, hipStream_t stream);
 
@@ -104,7 +112,7 @@ void launch_fill_zero(void* dst, size_t bytes, hipStream_t stream);
 // returns 0, or the non-zero status of the attention launch (shape not built, HIP error)
 int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
-                    float eps, int stages, hipStream_t stream);
+                    float eps, int stages, hipStream_t stream, int row0 = 0, int nrows = -1);
 
 // other widths / head shapes (triattn_generic.hip): head dim <= 64, C a multiple of 32
 size_t triattn_generic_blob_bytes(int C, int H);

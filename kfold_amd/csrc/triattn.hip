@@ -312,7 +312,12 @@ __global__ __launch_bounds__(512, 2) void triattn_out_kernel(
 // ------------------------------------------------------------------------------------------
 int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char* blob,
                     const TriattnWorkspace& ws, const void* residual, void* out, int N, int ending,
-                    float eps, int stages, hipStream_t stream) {
+                    float eps, int stages, hipStream_t stream, int row0, int nrows) {
+    // The input phase always covers all rows (the pair bias of a row is made from every row).  The
+    // attention and the output phase take the rows [row0, row0 + nrows) of x' (the transposed view
+    // for the ending node): a row is blockIdx.y / an entry of the row loop in every kernel, so a
+    // range is the same kernel entered row0 rows down its operands.
+    if (nrows < 0) { row0 = 0; nrows = N; }
     const int nb = (N + 31) / 32;
     bf16x8* qf = static_cast<bf16x8*>(ws.qf);
     bf16x8* kf = static_cast<bf16x8*>(ws.kf);
@@ -328,22 +333,32 @@ int launch_triattn(const void* x, int io_dtype, const uint8_t* mask, const char*
                                blob, qf, kf, vf, ws.biast, ws.codes, N, nb, ending, eps);
     }
 
+    if (nrows == 0) return 0;
+    const size_t row_frags = (size_t)kH * nb * 128;      // bf16x8 units of one row in q, k, v and o
     FlashArgs fa{};
-    fa.qf = qf; fa.kf = kf; fa.vf = vf; fa.gf = nullptr; fa.of = of;
-    fa.biast = ws.biast; fa.codes = ws.codes;
-    fa.nrows = N; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
+    fa.qf = qf + row0 * row_frags; fa.kf = kf + row0 * row_frags; fa.vf = vf + row0 * row_frags;
+    fa.gf = nullptr; fa.of = of + row0 * row_frags;
+    fa.biast = ws.biast; fa.codes = ws.codes + (size_t)row0 * nb * 32;
+    fa.nrows = nrows; fa.nb = nb; fa.H = kH; fa.bias_per_row = 0;
     if (stages & KFH_STAGE_CORE) {
-        const int rc = launch_flash(fa, 32, stream);
+        const int rc = launch_flash(fa, 32, stream, N);
         if (rc) return rc;
     }
     if (!(stages & KFH_STAGE_OUT)) return 0;
 
+    // position (row a, b) of x' is element (a * N + b) * C of x, or (b * N + a) * C for the ending node
+    const size_t esz = io_dtype == KFH_F32 ? 4 : 2;
+    const size_t shift = (ending ? (size_t)row0 : (size_t)row0 * N) * kC * esz;
+    const void* xr = static_cast<const char*>(x) + shift;
+    const void* rr = residual ? static_cast<const char*>(residual) + shift : nullptr;
+    void* outr = static_cast<char*>(out) + shift;
+    const dim3 grid_out((N + kTileA - 1) / kTileA, nrows);
     if (io_dtype == KFH_F32)
-        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_rows, dim3(512), 0, stream, of, x, blob,
-                           residual, out, N, nb, ending, eps);
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_F32>, grid_out, dim3(512), 0, stream, of + row0 * row_frags, xr, blob,
+                           rr, outr, N, nb, ending, eps);
     else
-        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_rows, dim3(512), 0, stream, of, x, blob,
-                           residual, out, N, nb, ending, eps);
+        hipLaunchKernelGGL(triattn_out_kernel<KFH_BF16>, grid_out, dim3(512), 0, stream, of + row0 * row_frags, xr, blob,
+                           rr, outr, N, nb, ending, eps);
     return 0;
 }
 

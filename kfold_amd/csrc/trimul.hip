@@ -290,8 +290,17 @@ __global__ __launch_bounds__(256, 3) void trimul_out_kernel(
 
 void launch_trimul_out(const uint16_t* planes_y, const void* z, const char* blob,
                        const void* residual, void* out, int io_dtype, int N, int Np, float eps,
-                       hipStream_t stream) {
-    dim3 grid((N + 127) / 128, N), block(256);
+                       hipStream_t stream, int row0, int nrows) {
+    // rows [row0, row0 + nrows) of the result: the kernel's row index is blockIdx.y, so the range is
+    // the same kernel entered row0 rows down every operand
+    if (nrows < 0) { row0 = 0; nrows = N; }
+    if (nrows == 0) return;
+    const size_t esz = io_dtype == KFH_F32 ? 4 : 2, shift = (size_t)row0 * N * kC * esz;
+    planes_y += (size_t)row0 * Np;
+    z = static_cast<const char*>(z) + shift;
+    if (residual) residual = static_cast<const char*>(residual) + shift;
+    out = static_cast<char*>(out) + shift;
+    dim3 grid((N + 127) / 128, nrows), block(256);
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL(trimul_out_kernel<KFH_F32>, grid, block, 0, stream, planes_y, z, blob,
                            residual, out, N, Np, eps);

@@ -268,9 +268,18 @@ int launch_trimul_in_wide(const void* z, int io_dtype, const uint8_t* mask, cons
 }
 
 int launch_trimul_out_wide(const uint16_t* planes_y, const void* z, const char* blob, const void* residual,
-                           void* out, int io_dtype, int N, int Np, int C, float eps, hipStream_t stream) {
+                           void* out, int io_dtype, int N, int Np, int C, float eps, hipStream_t stream,
+                           int row0, int nrows) {
     if (C != 256) return -1;
-    dim3 grid((N + 63) / 64, N), block(256);
+    if (nrows < 0) { row0 = 0; nrows = N; }
+    if (nrows == 0) return 0;
+    // rows [row0, row0 + nrows): blockIdx.y is the row, so every operand is entered row0 rows down
+    const size_t esz = io_dtype == KFH_F32 ? 4 : 2, shift = (size_t)row0 * N * C * esz;
+    planes_y += (size_t)row0 * Np;
+    z = static_cast<const char*>(z) + shift;
+    if (residual) residual = static_cast<const char*>(residual) + shift;
+    out = static_cast<char*>(out) + shift;
+    dim3 grid((N + 63) / 64, nrows), block(256);
     if (io_dtype == KFH_F32)
         hipLaunchKernelGGL((trimul_out_wide_kernel<KFH_F32, 256>), grid, block, 0, stream, planes_y, z, blob,
                            residual, out, N, Np, eps);

@@ -40,31 +40,47 @@ def _contiguous_io(t: torch.Tensor, name: str) -> None:
         raise TypeError(f"{name}: the hip block runs on bfloat16 or float32 tensors, got {t.dtype}")
 
 
-def _trimul_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor, before_write=None) -> None:
+def _trimul_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor, before_write=None,
+                    row_chunks: int = 1, side=None) -> None:
     params = _tm_parameters(mod)
     blob = cached_blob(mod, "_hip_multiplication_cache", cache_key(params, z, torch.bfloat16),
                        lambda: ops.trimul_pack(*params, device=z.device))
     ops.trimul_forward(z, mask, blob, mod.direction, eps=mod.layernorm_in.eps, residual=z, out=z,
-                       before_write=before_write)
+                       before_write=before_write, row_chunks=row_chunks, side=side)
 
 
-def _triattn_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor) -> None:
+def _triattn_inplace(mod: nn.Module, z: torch.Tensor, mask: torch.Tensor, row_chunks: int = 1, side=None) -> None:
     check_inf(mod)
     params = _ta_parameters(mod)
     blob = cached_blob(mod, "_hip_attention_cache", cache_key(params, z, torch.bfloat16),
                        lambda: ops.triattn_pack(*params, device=z.device))
     ops.triattn_forward(z, mask, blob, mod.no_heads, mod.starting, eps=mod.layer_norm.eps,
-                        residual=z, out=z)
+                        residual=z, out=z, row_chunks=row_chunks, side=side)
+
+
+def _phase_stream(holder: nn.Module, z: torch.Tensor):
+    """The second stream of a block that overlaps the phases of its ops (one per block and device)."""
+    if z.device.type != "cuda":
+        return None
+    cached = getattr(holder, "_hip_phase_stream", None)
+    if cached is None or cached[0] != z.device:
+        cached = (z.device, torch.cuda.Stream(z.device))
+        holder._hip_phase_stream = cached
+    return cached[1]
 
 
 class PairformerBlock(nn.Module):
     """tri-mul out, tri-mul in, tri-attn start, tri-attn end, transition(x2), final mask."""
 
     def __init__(self, channel_z: int = 128, num_tri_heads: int = 4, dropout: float = 0.1,
-                 kernel_backend: str = "hip"):
+                 kernel_backend: str = "hip", phase_row_chunks: int = 1):
         super().__init__()
         self.kernel_backend = kernel_backend
         self.channel_z = channel_z
+        # > 1: every triangle op runs its contraction / attention and its output phase over that many
+        # ranges of rows, the (memory-bound) output phase of a range on a second stream beside the
+        # (compute-bound) core phase of the next; results are the same bits (batch 1, c_z = 128)
+        self.phase_row_chunks = phase_row_chunks
         self.tri_mul_out = TriangleMultiplicationOutgoing(channel_z, kernel_backend=kernel_backend)
         self.tri_mul_in = TriangleMultiplicationIncoming(channel_z, kernel_backend=kernel_backend)
         self.tri_att_start = TriangleAttentionStartingNode(channel_z, num_tri_heads,
@@ -83,10 +99,12 @@ class PairformerBlock(nn.Module):
         if self.training:
             raise RuntimeError("The hip Pairformer block is inference-only (call .eval()).")
         _contiguous_io(z, "z")
-        _trimul_inplace(self.tri_mul_out, z, pair_mask, before_write=before_first_write)
-        _trimul_inplace(self.tri_mul_in, z, pair_mask)
-        _triattn_inplace(self.tri_att_start, z, pair_mask)
-        _triattn_inplace(self.tri_att_end, z, pair_mask)
+        k = self.phase_row_chunks
+        side = _phase_stream(self, z) if k > 1 else None
+        _trimul_inplace(self.tri_mul_out, z, pair_mask, before_write=before_first_write, row_chunks=k, side=side)
+        _trimul_inplace(self.tri_mul_in, z, pair_mask, row_chunks=k, side=side)
+        _triattn_inplace(self.tri_att_start, z, pair_mask, row_chunks=k, side=side)
+        _triattn_inplace(self.tri_att_end, z, pair_mask, row_chunks=k, side=side)
         return hip_transition(self.transition_z, z, residual=z, mask=pair_mask,
                               out=z if inplace_output else None)
 

@@ -83,6 +83,45 @@ def _batched_need(per_element: int, batched: int, given: torch.Tensor | None) ->
     return per_element
 
 
+def row_ranges(n: int, chunks: int, granule: int) -> list[tuple[int, int]]:
+    """[0, n) cut into at most ``chunks`` ranges (row0, nrows) that start at multiples of ``granule``
+    and are as even as the granule allows."""
+    blocks = (n + granule - 1) // granule
+    k = max(1, min(chunks, blocks))
+    out, b0 = [], 0
+    for c in range(k):
+        b1 = b0 + (blocks - b0) // (k - c)
+        r0, r1 = b0 * granule, min(b1 * granule, n)
+        out.append((r0, r1 - r0))
+        b0 = b1
+    return out
+
+
+def _run_phased(call, n: int, ranges, dev: torch.device, side, before_write=None) -> None:
+    """One op in phases over row ranges.  ``call(stages, row0, nrows)`` enqueues on the current
+    stream.  The input phase covers all rows; then the core phase of range c+1 (compute-bound) is
+    enqueued on the caller's stream while the output phase of range c (memory-bound) runs on ``side``.
+    Without ``side`` everything runs in order on the caller's stream.  Either way the kernels are those
+    of the whole op on offset pointers: same bits."""
+    call(_lib.KFH_STAGE_IN, 0, n)
+    if before_write is not None:
+        before_write()                         # the first output phase below writes
+    if side is None:
+        for r0, nr in ranges:
+            call(_lib.KFH_STAGE_CORE, r0, nr)
+            call(_lib.KFH_STAGE_OUT, r0, nr)
+        return
+    main = torch.cuda.current_stream(dev)
+    for r0, nr in ranges:
+        call(_lib.KFH_STAGE_CORE, r0, nr)
+        done = torch.cuda.Event()
+        done.record(main)
+        with torch.cuda.stream(side):
+            side.wait_event(done)
+            call(_lib.KFH_STAGE_OUT, r0, nr)
+    main.wait_stream(side)
+
+
 def workspace_bytes(op: str, **shape) -> int:
     """Bytes of scratch memory a forward call needs (0: shape not supported): ``trimul`` (N, C),
     ``triattn`` (N, C, heads) — both also with ``B``: the size that takes a batch through the kernels at
@@ -131,8 +170,13 @@ def trimul_pack(ln_in_w, ln_in_b, p_in_w, g_in_w, ln_out_w, ln_out_b, p_out_w, g
 def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, direction: str,
                    eps: float = 1e-5, residual: torch.Tensor | None = None,
                    out: torch.Tensor | None = None, before_write=None,
-                   workspace: torch.Tensor | None = None) -> torch.Tensor:
+                   workspace: torch.Tensor | None = None, row_chunks: int = 1,
+                   side: "torch.cuda.Stream | None" = None) -> torch.Tensor:
     """``out = (residual or 0) + TriangleMultiplication(z, mask)`` for z [*, N, N, C].
+
+    ``row_chunks`` > 1 (one batch element, C = 128 or 256): contraction and output phase run over
+    that many ranges of result rows, the output phase of a range on the stream ``side`` (if given)
+    beside the contraction of the next range; results are the same bits as with one range.
 
     ``workspace``: optional uint8 scratch tensor of at least ``workspace_bytes("trimul", N=, C=)``
     bytes to use instead of allocating one (its contents are overwritten).
@@ -166,8 +210,15 @@ def trimul_forward(z: torch.Tensor, mask: torch.Tensor, blob: torch.Tensor, dire
         ws_bytes = _batched_need(ws_bytes, L.kfh_trimul_workspace_bytes_batched(B, N, C), workspace)
     ws = _workspace(workspace, ws_bytes, dev)
     d = KFH_INCOMING if direction == "incoming" else KFH_OUTGOING
+    granule = L.kfh_trimul_row_granule(N, C) if row_chunks > 1 and B == 1 else 0
+    ranges = row_ranges(N, row_chunks, granule) if granule else []
     with torch.cuda.device(dev):
-        if before_write is None or B != 1:
+        if len(ranges) > 1:
+            head = (zc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual), out.data_ptr(),
+                    ws.data_ptr(), ws_bytes, B, N, C, d, float(eps), _io_dtype(zc))
+            _run_phased(lambda st, r0, nr: check(L.kfh_trimul_forward_rows(*head, st, r0, nr, _stream(dev))),
+                        N, ranges, dev, side, before_write)
+        elif before_write is None or B != 1:
             if before_write is not None:
                 before_write()
             check(L.kfh_trimul_forward(zc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
@@ -201,9 +252,11 @@ def triattn_pack(ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w, device: torch.devi
 
 def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tensor, heads: int,
                     starting: bool, eps: float = 1e-5, residual: torch.Tensor | None = None,
-                    out: torch.Tensor | None = None, workspace: torch.Tensor | None = None) -> torch.Tensor:
+                    out: torch.Tensor | None = None, workspace: torch.Tensor | None = None,
+                    row_chunks: int = 1, side: "torch.cuda.Stream | None" = None) -> torch.Tensor:
     """``out = (residual or 0) + TriangleAttention(x, mask)`` for x [*, N, N, C]; ``workspace`` as in
-    ``trimul_forward`` (``workspace_bytes("triattn", N=, C=, heads=)``)."""
+    ``trimul_forward`` (``workspace_bytes("triattn", N=, C=, heads=)``); ``row_chunks`` / ``side`` as in
+    ``trimul_forward`` (one batch element, C = 128 with 4 heads; ranges of 64 attention rows at least)."""
     dev = _require_cuda(x, mask, blob, residual, out)
     N, C = x.shape[-2], x.shape[-1]
     if x.dim() < 3 or x.shape[-3] != N:
@@ -231,10 +284,20 @@ def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tens
     if B > 1:
         ws_bytes = _batched_need(ws_bytes, L.kfh_triattn_workspace_bytes_batched(B, N, C, heads), workspace)
     ws = _workspace(workspace, ws_bytes, dev)
+    ranges = row_ranges(N, row_chunks, 64) if row_chunks > 1 and B == 1 and C == 128 and heads == 4 else []
+    if ranges and ranges[-1][1] < 48 and len(ranges) > 1:      # fold a short tail into the range before
+        (r0, nr), (_, tail) = ranges[-2], ranges[-1]
+        ranges[-2:] = [(r0, nr + tail)]
     with torch.cuda.device(dev):
-        check(L.kfh_triattn_forward(xc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
-                                    out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C, heads,
-                                    0 if starting else 1, float(eps), _io_dtype(xc), _stream(dev)))
+        if len(ranges) > 1:
+            head = (xc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual), out.data_ptr(),
+                    ws.data_ptr(), ws_bytes, B, N, C, heads, 0 if starting else 1, float(eps), _io_dtype(xc))
+            _run_phased(lambda st, r0, nr: check(L.kfh_triattn_forward_rows(*head, st, r0, nr, _stream(dev))),
+                        N, ranges, dev, side)
+        else:
+            check(L.kfh_triattn_forward(xc.data_ptr(), m8.data_ptr(), blob.data_ptr(), _ptr(residual),
+                                        out.data_ptr(), ws.data_ptr(), ws_bytes, B, N, C, heads,
+                                        0 if starting else 1, float(eps), _io_dtype(xc), _stream(dev)))
     return out
 
 

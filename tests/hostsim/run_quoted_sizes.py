@@ -13,6 +13,7 @@ from __future__ import annotations
 import sys
 import time
 
+import tests.test_block_gpu as BK
 import tests.test_quoted_sizes_gpu as Q
 import tests.test_shipping_dims_gpu as SD
 import tests.test_triattn_gpu as TA
@@ -30,6 +31,7 @@ CASES = [
     (TA, "test_triattn_config3_n512", [(True,), (False,)]),
     (SD, "test_triattn_c64_templates_n384", [(True,), (False,)]),
     (SD, "test_trimul_c256_tiled_sizes", [("outgoing", 384), ("incoming", 384), ("outgoing", 768), ("incoming", 768)]),
+    (BK, "test_phases_over_row_ranges_at_the_benchmark_size", [()]),
 ]
 
 

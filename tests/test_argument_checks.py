@@ -58,6 +58,18 @@ def test_trimul_argument_checks(env):
     # the stage-selective variant checks the same things
     s = lib.kfh_trimul_forward_stages
     _expect(lib, s(p[0], p[1], p[2], None, p[3], p[4], 0, 1, 64, 128, 0, 1e-5, 0, 7, None), EINVAL, "workspace")
+    # ranges of rows: tile-aligned, one batch element, the fused widths
+    r = lib.kfh_trimul_forward_rows
+    assert lib.kfh_trimul_row_granule(768, 128) == 256 and lib.kfh_trimul_row_granule(300, 256) == 128
+    assert lib.kfh_trimul_row_granule(300, 64) == 0 and lib.kfh_trimul_row_granule(0, 128) == 0
+    big = lib.kfh_trimul_workspace_bytes(768, 128)
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 128, 0, 1e-5, 0, 6, 100, 256, None), EINVAL,
+            "multiples of 256")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 128, 0, 1e-5, 0, 6, 256, 100, None), EINVAL, "rows [256, 356)")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 128, 0, 1e-5, 0, 6, 512, 512, None), EINVAL, "of 768")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 2, 768, 128, 0, 1e-5, 0, 6, 0, 256, None), EUNSUPPORTED, "B = 1")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 64, 0, 1e-5, 0, 6, 0, 256, None), EUNSUPPORTED, "C = 128 or 256")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], 0, 1, 768, 128, 0, 1e-5, 0, 6, 256, 512, None), EINVAL, "workspace")
 
 
 def test_triattn_argument_checks(env):
@@ -75,6 +87,13 @@ def test_triattn_argument_checks(env):
     _expect(lib, f(p[0], p[1], p[2], None, p[0], p[4], need, 1, 64, 128, 4, 1, 1e-5, 0, None), EINVAL, "alias")
     _expect(lib, f(p[0], p[1], p[2], p[0], p[0], p[4], need - 1, 1, 64, 128, 4, 1, 1e-5, 0, None), EINVAL, "workspace")
     _expect(lib, f(p[0], p[1], p[2], None, p[3], p[4], 16, 2, 64, 64, 4, 0, 1e-5, 0, None), EINVAL, "workspace")
+    r = lib.kfh_triattn_forward_rows
+    big = lib.kfh_triattn_workspace_bytes(768, 128, 4)
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 128, 4, 0, 1e-5, 0, 6, 700, 100, None), EINVAL, "rows [700, 800)")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 128, 4, 0, 1e-5, 0, 6, -1, 100, None), EINVAL, "rows")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 2, 768, 128, 4, 0, 1e-5, 0, 6, 0, 100, None), EUNSUPPORTED, "B = 1")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], big, 1, 768, 64, 4, 0, 1e-5, 0, 6, 0, 100, None), EUNSUPPORTED, "C = 128")
+    _expect(lib, r(p[0], p[1], p[2], None, p[3], p[4], 0, 1, 768, 128, 4, 0, 1e-5, 0, 6, 0, 100, None), EINVAL, "workspace")
     g = lib.kfh_triattn_pack
     _expect(lib, g(*p[:8], 0, 128, 3, p[8], None), EUNSUPPORTED, "H=3")
     _expect(lib, g(*p[:8], 9, 128, 4, p[8], None), EINVAL, "w_dtype")

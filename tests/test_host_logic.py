@@ -20,7 +20,7 @@ class Recorder:
 
     def __getattr__(self, name):
         res, argtypes = self.signatures[name]              # KeyError: not in the header
-        if name.endswith("_bytes") or name in ("kfh_version", "kfh_last_error"):
+        if name.endswith(("_bytes", "_granule")) or name in ("kfh_version", "kfh_last_error"):
             return getattr(self.real, name)
 
         def call(*args):
@@ -377,3 +377,39 @@ def test_transition_rows_and_mask_plumbing(rec):
         wide(s)
     c = rec.of("kfh_transition_forward")[1]
     assert (c[7], c[8], c[9], c[11]) == (30, 384, 4, 0) and c[5] and c[6] > 0
+
+
+def test_block_with_phases_over_row_ranges(rec):
+    """phase_row_chunks = 2 at N = 300 (contraction tiles of 128 rows): every triangle op becomes one
+    input phase over all rows, then core and output phase per range, in place on z; the transition
+    and the default block are untouched."""
+    from kfold_amd import _lib, modules
+
+    N = 300
+    blk = modules.PairformerBlock(phase_row_chunks=2).eval()
+    z = torch.zeros(1, N, N, 128, dtype=torch.bfloat16)
+    pair = torch.ones(1, N, N, dtype=torch.bool)
+    waits = []
+    with torch.no_grad():
+        blk(z, pair, inplace_output=True, before_first_write=lambda: waits.append(len(rec.calls)))
+    IN, CORE, OUT = _lib.KFH_STAGE_IN, _lib.KFH_STAGE_CORE, _lib.KFH_STAGE_OUT
+    tm = rec.of("kfh_trimul_forward_rows")
+    assert [(c[13], c[14], c[15]) for c in tm] == 2 * [(IN, 0, N), (CORE, 0, 128), (OUT, 0, 128),
+                                                       (CORE, 128, 172), (OUT, 128, 172)]
+    assert all(c[0] == c[3] == c[4] == z.data_ptr() and c[7] == 1 for c in tm)
+    assert [c[10] for c in tm] == 5 * [0] + 5 * [1]                       # outgoing, then incoming
+    ta = rec.of("kfh_triattn_forward_rows")
+    assert [(c[14], c[15], c[16]) for c in ta] == 2 * [(IN, 0, N), (CORE, 0, 128), (OUT, 0, 128),
+                                                       (CORE, 128, 172), (OUT, 128, 172)]
+    assert [c[11] for c in ta] == 5 * [0] + 5 * [1]                       # starting, then ending node
+    assert rec.names(("_forward", "_forward_stages")) == ["kfh_transition_forward"]
+    # the caller's wait is placed after the input phase of the first op and before its first output phase
+    first_in = next(i for i, (n, a) in enumerate(rec.calls) if n == "kfh_trimul_forward_rows")
+    assert waits == [first_in + 1]
+    # a range shorter than the attention kernel takes: the op runs in one piece
+    rec.calls.clear()
+    small = torch.zeros(1, 70, 70, 128, dtype=torch.bfloat16)
+    with torch.no_grad():
+        blk(small, torch.ones(1, 70, 70, dtype=torch.bool), inplace_output=True)
+    assert rec.names(("_forward",)) == ["kfh_trimul_forward", "kfh_trimul_forward", "kfh_triattn_forward",
+                                        "kfh_triattn_forward", "kfh_transition_forward"]
