@@ -54,6 +54,25 @@ def test_walk_pair_block(n):
     assert launches > 0
 
 
+@pytest.mark.parametrize("n,chunks", [(768, 3), (1000, 4), (1280, 3)])
+def test_walk_pair_block_in_row_ranges(n, chunks):
+    """The same block with every triangle op's core and output phase run over ranges of rows (offset
+    pointers into planes, fragments, key codes, z): strip attention kernel at 768 and 1000 (N = 1000
+    is no multiple of the 32-row blocks or the 128-row tiles), staged kernel at 1280."""
+    from kfold_amd import modules as M
+
+    blk = M.PairformerBlock(phase_row_chunks=chunks).eval()
+    synthetic.init_weights_(blk, 0)
+    tok = synthetic.token_mask(n, synthetic.n_pad_for(n, 0.12))
+    pm = synthetic.pair_mask_from_tokens(tok)
+    with torch.no_grad(), _walk(stride=211) as arena:
+        z = arena.like(_pattern((1, n, n, 128)))
+        before = hostsim.load().hostsim_launch_count()
+        blk(z, arena.like(pm), inplace_output=True)
+        # input phase + (core, output) per range for the four ops, and the transition
+        assert hostsim.load().hostsim_launch_count() - before >= 4 * (1 + 2 * chunks) + 1
+
+
 @pytest.mark.parametrize("n", [768, 1280])
 def test_walk_triangular_block_c256(n):
     """Shipping trunk block: tri-mul at C = 256 (both directions) + transition x4."""
