@@ -443,10 +443,62 @@ def case_api(r, g, dev, arena=None):
     return what, {"max_abs": 0.0, "rel_fro": 0.0}
 
 
+def case_ranges(r, g, dev):
+    """Core and output phase over ranges of rows against the op in one piece: same bits, for random
+    sizes (not multiples of the tiles), range counts, directions / nodes, dtypes, in place or not."""
+    from kfold_amd import ops, primitives as P
+
+    dtype = r.choice([torch.bfloat16, torch.float32])
+    inplace = r.random() < 0.5
+    if r.random() < 0.5:
+        c = r.choice([128, 256])
+        n = r.randint(257, 384)                     # planes of 384 rows: three tile rows of 128
+        incoming = r.random() < 0.5
+        chunks = r.randint(2, 4)
+        what = f"ranges trimul C={c} N={n} incoming={incoming} chunks={chunks} {dtype} inplace={inplace}"
+        cls = "TriangleMultiplicationIncoming" if incoming else "TriangleMultiplicationOutgoing"
+        mod = synthetic.init_weights_(getattr(P, cls)(c).eval(), r.randrange(100), std=0.05).to(dev)
+        x = torch.randn(1, n, n, c, generator=g).to(dtype).to(dev)
+        mask = _pair_mask(r, g, 1, n).to(dev)
+        with torch.no_grad():
+            mod(x[:, :4, :4].contiguous(), mask[:, :4, :4].contiguous())
+            blob, d = mod._hip_multiplication_cache, mod.direction
+            if inplace:
+                a, b = x.clone(), x.clone()
+                ops.trimul_forward(a, mask, blob, d, residual=a, out=a)
+                ops.trimul_forward(b, mask, blob, d, residual=b, out=b, row_chunks=chunks)
+            else:
+                a = ops.trimul_forward(x, mask, blob, d)
+                b = ops.trimul_forward(x, mask, blob, d, row_chunks=chunks)
+        assert torch.equal(a, b), what
+        return what, {"max_abs": 0.0, "rel_fro": 0.0}
+    n = r.randint(129, 300)
+    starting = r.random() < 0.5
+    chunks = r.randint(2, 4)
+    what = f"ranges triattn N={n} starting={starting} chunks={chunks} {dtype} inplace={inplace}"
+    cls = "TriangleAttentionStartingNode" if starting else "TriangleAttentionEndingNode"
+    mod = synthetic.init_weights_(getattr(P, cls)(128, 4).eval(), r.randrange(100), std=0.08).to(dev)
+    x = torch.randn(1, n, n, 128, generator=g).to(dtype).to(dev)
+    mask = _pair_mask(r, g, 1, n).to(dev)
+    with torch.no_grad():
+        mod(x[:, :4, :4].contiguous(), mask[:, :4, :4].contiguous())
+        blob = mod._hip_attention_cache
+        if inplace:
+            a, b = x.clone(), x.clone()
+            ops.triattn_forward(a, mask, blob, 4, starting, residual=a, out=a)
+            ops.triattn_forward(b, mask, blob, 4, starting, residual=b, out=b, row_chunks=chunks)
+        else:
+            a = ops.triattn_forward(x, mask, blob, 4, starting)
+            b = ops.triattn_forward(x, mask, blob, 4, starting, row_chunks=chunks)
+    assert torch.equal(a, b), what
+    return what, {"max_abs": 0.0, "rel_fro": 0.0}
+
+
 FAMILIES = {
     "trimul": case_trimul, "triattn": case_triattn, "transition": case_transition, "apb": case_apb,
     "cross": case_cross, "parcae": case_parcae, "block": case_block,
     "wide_block": case_wide_block, "template_block": case_template_block, "api": case_api,
+    "ranges": case_ranges,
 }
 _ORDER = ["trimul", "triattn", "transition", "apb", "cross", "parcae", "block", "trimul", "triattn", "apb"]
 
