@@ -72,3 +72,14 @@ def test_host_model_vectors_are_current():
     with hostsim.host_backend():
         stats = compare(hostsim.HostDevice("cpu"))
     assert all(frac == 1.0 for frac, _ in stats.values()), stats
+
+
+def test_smoke_body_on_the_host_build(capsys):
+    """What __graft_entry__.smoke() runs on cuda:0, run on the kernels' host build: the call sequence,
+    the oracle comparison and its thresholds."""
+    import __graft_entry__ as entry
+    from tests import hostsim
+
+    with hostsim.host_backend():
+        entry._smoke_on(hostsim.HostDevice("cpu"))
+    assert "smoke ok" in capsys.readouterr().out
