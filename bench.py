@@ -188,14 +188,14 @@ def cpu_baseline(n: int) -> dict:
 class Harness:
     """One block's modules, inputs and stage-selective launches for the per-kernel timings."""
 
-    def __init__(self, n: int, pad_frac: float, std: float = 0.02, seed: int = 0):
+    def __init__(self, n: int, pad_frac: float, std: float = 0.02, seed: int = 0, dev=None):
         import torch
 
         from kfold_amd import _lib, modules, synthetic
 
         self.torch, self._lib = torch, _lib
         self.L = _lib.lib()
-        self.dev = torch.device("cuda:0")
+        self.dev = torch.device("cuda:0") if dev is None else dev
         self.n, self.n_pad = n, synthetic.n_pad_for(n, pad_frac)
         self.block = modules.PairSingleBlock().eval()
         synthetic.init_weights_(self.block, seed, std=std)

@@ -83,3 +83,23 @@ def test_smoke_body_on_the_host_build(capsys):
     with hostsim.host_backend():
         entry._smoke_on(hostsim.HostDevice("cpu"))
     assert "smoke ok" in capsys.readouterr().out
+
+
+def test_per_kernel_table_on_the_host_build(monkeypatch):
+    """bench.py's harness (stage-selective launches of one block's kernels) and its per-kernel table at
+    a small size on the host build; the times are stand-ins."""
+    import bench
+    from tests import hostsim
+
+    monkeypatch.setattr(bench, "event_time_ms", lambda fn, iters, warm=2: [(fn(), 1.0)[1]] * 2)
+    import torch
+
+    with hostsim.host_backend(), torch.inference_mode():        # as bench.main() calls them
+        h = bench.Harness(40, 0.12, dev=hostsim.HostDevice("cpu"))
+        assert h.flash_ms(2) == 1.0
+        table = bench.per_kernel_table(h, {"kfh::flash_strip_kernel": (10.0, 5.0)}, iters=2)
+    assert set(table) == {"trimul_in_kernel", "contract_kernel", "trimul_out_kernel", "triattn_proj_kernel",
+                          "flash_strip_kernel", "triattn_out_kernel", "transition_kernel", "pair_bias_kernel"}
+    assert table["flash_strip_kernel"]["measured_MB"] == 15.0 and table["contract_kernel"]["measured_MB"] is None
+    assert bench.flash_executed_flops(h.pm, 40) > 0
+    assert bench.block_flops(768)["block"] > 1.2e12
