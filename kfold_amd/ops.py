@@ -241,7 +241,7 @@ def triattn_pack(ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w, device: torch.devi
     C, H = q_w.shape[1], bias_w.shape[0]
     nbytes = L.kfh_triattn_packed_bytes(C, H)
     if nbytes == 0:
-        raise NotImplementedError(f"hip triangle attention is built for C=128, H=4; got C={C}, H={H}")
+        raise NotImplementedError(f"hip triangle attention takes C a multiple of 32 and head dim <= 64; got C={C}, H={H}")
     ws = _weights_f32(device, ln_w, ln_b, q_w, k_w, v_w, g_w, bias_w, o_w)
     blob = torch.empty(nbytes, dtype=torch.uint8, device=device)
     with torch.cuda.device(device):
@@ -280,7 +280,7 @@ def triattn_forward(x: torch.Tensor, mask: torch.Tensor | None, blob: torch.Tens
     ws_bytes = L.kfh_triattn_workspace_bytes(N, C, heads)
     if ws_bytes == 0:
         raise NotImplementedError(
-            f"hip triangle attention is built for C=128, H=4, N<=8192; got C={C}, H={heads}, N={N}")
+            f"hip triangle attention takes C a multiple of 32, head dim <= 64, N <= 8192; got C={C}, H={heads}, N={N}")
     if B > 1:
         ws_bytes = _batched_need(ws_bytes, L.kfh_triattn_workspace_bytes_batched(B, N, C, heads), workspace)
     ws = _workspace(workspace, ws_bytes, dev)
