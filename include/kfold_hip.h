@@ -336,6 +336,24 @@ int kfh_parcae_pack(const void* ln_w, const void* ln_b, const void* log_a, const
 int kfh_parcae_step(const void* z, const void* u, const void* u_add, const void* blob, void* out,
                     long long rows, int C, float eps, int io_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * The pair track of one Pairformer block in one call (modules/apo_module.py:145-172, eval mode):
+ *   z += TriMulOut(z, m); z += TriMulIn(z, m); z += TriAttStart(z, m); z += TriAttEnd(z, m);
+ *   z  = (z + Transition(z)) * m
+ * in place on z [B, N, N, C] with pair_mask [B, N, N] (bytes), the five blobs from kfh_trimul_pack
+ * (outgoing, incoming), kfh_triattn_pack (starting, ending node) and kfh_transition_pack, and one
+ * workspace of kfh_pair_block_workspace_bytes() bytes shared by the five ops (they run one after the
+ * other on `stream`).  Same kernels and bits as the five calls made separately; supported shapes are
+ * those all three ops support (C = 128 with 4 heads fused; other multiples of 32 up to 256 through
+ * the assembled paths).
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_pair_block_workspace_bytes(int B, int N, int C, int H, int expansion);
+int kfh_pair_block_forward(void* z, const uint8_t* pair_mask, const void* trimul_out_blob,
+                           const void* trimul_in_blob, const void* triattn_start_blob,
+                           const void* triattn_end_blob, const void* transition_blob, void* workspace,
+                           size_t workspace_bytes, int B, int N, int C, int H, int expansion, float eps,
+                           int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -353,4 +353,44 @@ int kfh_triattn_forward_rows(const void* x, const uint8_t* mask, const void* blo
     return check_launch("triattn_forward");
 }
 
+size_t kfh_pair_block_workspace_bytes(int B, int N, int C, int H, int expansion) {
+    if (B <= 0) return 0;
+    // the sizes that take a batch through the kernels at once where the path can
+    const size_t a = kfh_trimul_workspace_bytes_batched(B, N, C), b = kfh_triattn_workspace_bytes_batched(B, N, C, H);
+    if (a == 0 || b == 0 || kfh_transition_packed_bytes(C, expansion) == 0) return 0;
+    const size_t c = kfh_transition_workspace_bytes((long long)B * N * N, C, expansion);
+    return a > b ? (a > c ? a : c) : (b > c ? b : c);
+}
+
+int kfh_pair_block_forward(void* z, const uint8_t* pair_mask, const void* trimul_out_blob,
+                           const void* trimul_in_blob, const void* triattn_start_blob,
+                           const void* triattn_end_blob, const void* transition_blob, void* workspace,
+                           size_t workspace_bytes, int B, int N, int C, int H, int expansion, float eps,
+                           int io_dtype, void* stream) {
+    const size_t need = kfh_pair_block_workspace_bytes(B > 0 ? B : 1, N, C, H, expansion);
+    if (need == 0)
+        return fail(KFH_EUNSUPPORTED, "pair_block_forward: C=%d H=%d expansion=%d N=%d not supported", C, H, expansion, N);
+    if (B <= 0) return fail(KFH_EINVAL, "pair_block_forward: bad shape B=%d N=%d", B, N);
+    if (!z || !pair_mask || !trimul_out_blob || !trimul_in_blob || !triattn_start_blob || !triattn_end_blob ||
+        !transition_blob || !workspace)
+        return fail(KFH_EINVAL, "pair_block_forward: null pointer argument");
+    if (workspace_bytes < need)
+        return fail(KFH_EINVAL, "pair_block_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+    // the five in-place updates of the reference's eval-mode block, each with its residual fused
+    int rc = kfh_trimul_forward(z, pair_mask, trimul_out_blob, z, z, workspace, workspace_bytes, B, N, C,
+                                KFH_OUTGOING, eps, io_dtype, stream);
+    if (rc) return rc;
+    rc = kfh_trimul_forward(z, pair_mask, trimul_in_blob, z, z, workspace, workspace_bytes, B, N, C, KFH_INCOMING,
+                            eps, io_dtype, stream);
+    if (rc) return rc;
+    rc = kfh_triattn_forward(z, pair_mask, triattn_start_blob, z, z, workspace, workspace_bytes, B, N, C, H, 0, eps,
+                             io_dtype, stream);
+    if (rc) return rc;
+    rc = kfh_triattn_forward(z, pair_mask, triattn_end_blob, z, z, workspace, workspace_bytes, B, N, C, H, 1, eps,
+                             io_dtype, stream);
+    if (rc) return rc;
+    return kfh_transition_forward(z, transition_blob, z, pair_mask, z, workspace, workspace_bytes,
+                                  (long long)B * N * N, C, expansion, eps, io_dtype, stream);
+}
+
 }  // extern "C"

@@ -197,3 +197,19 @@ def test_window_attention_and_recurrence_argument_checks(env):
     h = lib.kfh_parcae_pack
     _expect(lib, h(p[0], p[1], p[2], p[3], p[4], 0, 64, p[5], None), EUNSUPPORTED, "C=64")
     _expect(lib, h(p[0], p[1], None, p[3], p[4], 0, 128, p[5], None), EINVAL, "null")
+
+
+def test_pair_block_argument_checks(env):
+    lib, p, _ = env
+    need = lib.kfh_pair_block_workspace_bytes(1, 64, 128, 4, 2)
+    assert need == max(lib.kfh_trimul_workspace_bytes(64, 128), lib.kfh_triattn_workspace_bytes(64, 128, 4))
+    assert lib.kfh_pair_block_workspace_bytes(3, 40, 64, 4, 2) >= lib.kfh_triattn_workspace_bytes_batched(3, 40, 64, 4)
+    assert lib.kfh_pair_block_workspace_bytes(0, 64, 128, 4, 2) == 0
+    f = lib.kfh_pair_block_forward
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need, 1, 64, 48, 4, 2, 1e-5, 0, None), EUNSUPPORTED, "C=48")
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need, 1, 64, 128, 3, 2, 1e-5, 0, None), EUNSUPPORTED, "H=3")
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need, 0, 64, 128, 4, 2, 1e-5, 0, None), EINVAL, "B=0")
+    _expect(lib, f(p[0], p[1], p[2], p[3], None, p[5], p[6], p[7], need, 1, 64, 128, 4, 2, 1e-5, 0, None), EINVAL, "null")
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need - 1, 1, 64, 128, 4, 2, 1e-5, 0, None), EINVAL,
+            "workspace", str(need))
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need, 1, 64, 128, 4, 2, 1e-5, 9, None), EINVAL, "io_dtype")

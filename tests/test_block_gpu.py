@@ -296,3 +296,37 @@ def _check_row_ranges(n, widths, trimul_chunks, triattn_chunks, both=True):
                     if on_gpu:
                         torch.cuda.synchronize()
                     assert torch.equal(parts, whole), f"tri-attn {cls} {dtype} in {chunks} ranges"
+
+
+@pytest.mark.parametrize("c,heads,batch,n", [(128, 4, 1, 70), (128, 4, 2, 37), (64, 4, 3, 45)])
+def test_pair_block_in_one_c_call(c, heads, batch, n):
+    """kfh_pair_block_forward (the pair track of a block in one C call, for callers without the Python
+    layer) against the module: same kernels, same bits; fp32 and bf16 tensors."""
+    from kfold_amd import _lib, modules as M
+
+    print(f"case pair block in one C call c={c} batch={batch} n={n}", flush=True)
+    blk = synthetic.init_weights_(M.PairformerBlock(c, heads).eval(), 4, std=0.05).to(DEV)
+    g = torch.Generator().manual_seed(n)
+    pm = torch.stack([synthetic.pair_mask_from_tokens(synthetic.token_mask(n, 3 * b))[0] for b in range(batch)]).to(DEV)
+    L = _lib.lib()
+    for dtype in (torch.bfloat16, torch.float32):
+        z = torch.randn(batch, n, n, c, generator=g).to(dtype).to(DEV)
+        with torch.no_grad():
+            want = blk(z.clone(), pm, inplace_output=True)
+        blobs = [blk.tri_mul_out._hip_multiplication_cache, blk.tri_mul_in._hip_multiplication_cache,
+                 blk.tri_att_start._hip_attention_cache, blk.tri_att_end._hip_attention_cache,
+                 blk.transition_z._hip_transition_cache]
+        need = L.kfh_pair_block_workspace_bytes(batch, n, c, heads, 2)
+        assert need > 0
+        ws = torch.empty(need + 256, dtype=torch.uint8, device=DEV)
+        ws = ws[(-ws.data_ptr()) % 256:][:need]
+        got = z.clone()
+        m8 = pm.contiguous().view(torch.uint8)
+        io = _lib.KFH_BF16 if dtype == torch.bfloat16 else _lib.KFH_F32
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(L.kfh_pair_block_forward(got.data_ptr(), m8.data_ptr(), *[b.data_ptr() for b in blobs], ws.data_ptr(),
+                                            need, batch, n, c, heads, 2, 1e-5, io, stream))
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"{dtype}"
+        assert (got.float().cpu()[~pm.cpu()] == 0).all()
+    assert L.kfh_pair_block_workspace_bytes(1, n, 48, 4, 2) == 0
