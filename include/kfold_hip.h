@@ -354,6 +354,19 @@ int kfh_pair_block_forward(void* z, const uint8_t* pair_mask, const void* trimul
                            size_t workspace_bytes, int B, int N, int C, int H, int expansion, float eps,
                            int io_dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------
+ * The single track that follows the pair track (modules/confidence_head.py:161-175, eval mode):
+ *   bias = linear_pair_bias(LN(z));  s += SelfAttentionPairBias(s, None, bias, mask);  s += Transition(s)
+ * in place on s [B, N, Cs]; z [B, N, N, Cz] is only read; token_mask [B, N] (bytes).  Blobs from
+ * kfh_pair_bias_pack, kfh_apb_pack (unconditioned, bf16 arithmetic) and kfh_transition_pack.  The
+ * workspace also holds the bias tiles.  Same kernels and bits as the three calls made separately.
+ * ------------------------------------------------------------------------------------- */
+size_t kfh_single_track_workspace_bytes(int B, int N, int Cz, int Cs, int H, int expansion);
+int kfh_single_track_forward(const void* z, void* s, const uint8_t* token_mask, const void* pair_bias_blob,
+                             const void* apb_blob, const void* transition_blob, void* workspace,
+                             size_t workspace_bytes, int B, int N, int Cz, int Cs, int H, int expansion,
+                             float eps, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,9 @@ SIGNATURES: dict[str, tuple] = {
                                           c_float, c_int, c_int, _P]),
     "kfh_triattn_forward_stages": (c_int, [_P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int,
                                            c_int, c_float, c_int, c_int, _P]),
+    "kfh_single_track_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "kfh_single_track_forward": (c_int, [_P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int,
+                                         c_int, c_float, c_int, _P]),
     "kfh_pair_block_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "kfh_pair_block_forward": (c_int, [_P, _P, _P, _P, _P, _P, _P, _P, c_size_t, c_int, c_int, c_int, c_int, c_int,
                                        c_float, c_int, _P]),

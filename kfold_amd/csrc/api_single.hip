@@ -498,4 +498,37 @@ int kfh_transition_forward_static(const void* x, const void* blob, const void* r
                                    io_dtype, stream);
 }
 
+size_t kfh_single_track_workspace_bytes(int B, int N, int Cz, int Cs, int H, int expansion) {
+    const size_t tiles = kfh_bias_tiles_bytes(B, H, N, KFH_ARITH_BF16);
+    const size_t att = kfh_apb_workspace_bytes(B, N, Cs, H, 0, KFH_ARITH_BF16);
+    if (Cz != kC || tiles == 0 || att == 0 || kfh_transition_packed_bytes(Cs, expansion) == 0) return 0;
+    const size_t tr = kfh_transition_workspace_bytes((long long)B * N, Cs, expansion);
+    return tiles + (att > tr ? att : tr);
+}
+
+int kfh_single_track_forward(const void* z, void* s, const uint8_t* token_mask, const void* pair_bias_blob,
+                             const void* apb_blob, const void* transition_blob, void* workspace,
+                             size_t workspace_bytes, int B, int N, int Cz, int Cs, int H, int expansion,
+                             float eps, int io_dtype, void* stream) {
+    if (B <= 0 || N <= 0) return fail(KFH_EINVAL, "single_track_forward: bad shape B=%d N=%d", B, N);
+    const size_t need = kfh_single_track_workspace_bytes(B, N, Cz, Cs, H, expansion);
+    if (need == 0)
+        return fail(KFH_EUNSUPPORTED, "single_track_forward: Cz=%d Cs=%d H=%d expansion=%d N=%d not supported", Cz, Cs,
+                    H, expansion, N);
+    if (!z || !s || !token_mask || !pair_bias_blob || !apb_blob || !transition_blob || !workspace)
+        return fail(KFH_EINVAL, "single_track_forward: null pointer argument");
+    if (workspace_bytes < need)
+        return fail(KFH_EINVAL, "single_track_forward: workspace %zu < %zu bytes", workspace_bytes, need);
+    char* ws = static_cast<char*>(workspace);
+    const size_t tiles = kfh_bias_tiles_bytes(B, H, N, KFH_ARITH_BF16);
+    // pair bias of every batch element from z, attention with it (s += ...), transition (s += ...)
+    int rc = kfh_pair_bias_project(z, pair_bias_blob, ws, B, N, Cz, H, eps, io_dtype, stream);
+    if (rc) return rc;
+    rc = kfh_apb_forward(s, nullptr, ws, token_mask, apb_blob, s, s, ws + tiles, workspace_bytes - tiles, B, N, Cs, H, 0,
+                         1, B > 1, B > 1, 0, eps, io_dtype, KFH_ARITH_BF16, stream);
+    if (rc) return rc;
+    return kfh_transition_forward(s, transition_blob, s, nullptr, s, ws + tiles, workspace_bytes - tiles,
+                                  (long long)B * N, Cs, expansion, eps, io_dtype, stream);
+}
+
 }  // extern "C"

@@ -213,3 +213,17 @@ def test_pair_block_argument_checks(env):
     _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need - 1, 1, 64, 128, 4, 2, 1e-5, 0, None), EINVAL,
             "workspace", str(need))
     _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], p[7], need, 1, 64, 128, 4, 2, 1e-5, 9, None), EINVAL, "io_dtype")
+
+
+def test_single_track_argument_checks(env):
+    lib, p, _ = env
+    need = lib.kfh_single_track_workspace_bytes(1, 64, 128, 384, 16, 4)
+    assert need >= lib.kfh_bias_tiles_bytes(1, 16, 64, 0) + lib.kfh_apb_workspace_bytes(1, 64, 384, 16, 0, 0)
+    assert lib.kfh_single_track_workspace_bytes(1, 64, 256, 384, 16, 4) == 0       # pair bias is built for c_z = 128
+    f = lib.kfh_single_track_forward
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], need, 1, 64, 256, 384, 16, 4, 1e-5, 0, None), EUNSUPPORTED, "Cz=256")
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], need, 1, 64, 128, 384, 5, 4, 1e-5, 0, None), EUNSUPPORTED, "H=5")
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], need, 0, 64, 128, 384, 16, 4, 1e-5, 0, None), EINVAL, "B=0")
+    _expect(lib, f(p[0], None, p[2], p[3], p[4], p[5], p[6], need, 1, 64, 128, 384, 16, 4, 1e-5, 0, None), EINVAL, "null")
+    _expect(lib, f(p[0], p[1], p[2], p[3], p[4], p[5], p[6], need - 1, 1, 64, 128, 384, 16, 4, 1e-5, 0, None), EINVAL,
+            "workspace", str(need))

@@ -330,3 +330,35 @@ def test_pair_block_in_one_c_call(c, heads, batch, n):
         assert torch.equal(got, want), f"{dtype}"
         assert (got.float().cpu()[~pm.cpu()] == 0).all()
     assert L.kfh_pair_block_workspace_bytes(1, n, 48, 4, 2) == 0
+
+
+@pytest.mark.parametrize("batch,n", [(1, 70), (2, 37)])
+def test_single_track_in_one_c_call(batch, n):
+    """kfh_single_track_forward (pair bias from z, attention, transition, in place on s) against the
+    module's single track: same kernels, same bits."""
+    from kfold_amd import _lib, modules as M
+
+    print(f"case single track in one C call batch={batch} n={n}", flush=True)
+    blk = synthetic.init_weights_(M.PairSingleBlock().eval(), 7, std=0.05).to(DEV)
+    g = torch.Generator().manual_seed(n)
+    tok = torch.stack([synthetic.token_mask(n, 4 * b)[0] for b in range(batch)]).to(DEV)
+    L = _lib.lib()
+    for dtype in (torch.bfloat16, torch.float32):
+        z = torch.randn(batch, n, n, 128, generator=g).to(dtype).to(DEV)
+        s = torch.randn(batch, n, 384, generator=g).to(dtype).to(DEV)
+        want = s.clone()
+        with torch.no_grad():
+            blk.single_track(z, want, tok)
+        blobs = [blk._hip_pair_bias_cache, blk.attention._hip_apb_cache, blk.transition._hip_transition_cache]
+        need = L.kfh_single_track_workspace_bytes(batch, n, 128, 384, 16, 4)
+        assert need > 0
+        ws = torch.empty(need + 256, dtype=torch.uint8, device=DEV)
+        ws = ws[(-ws.data_ptr()) % 256:][:need]
+        got = s.clone()
+        io = _lib.KFH_BF16 if dtype == torch.bfloat16 else _lib.KFH_F32
+        _lib.check(L.kfh_single_track_forward(z.data_ptr(), got.data_ptr(), tok.contiguous().view(torch.uint8).data_ptr(),
+                                              *[b.data_ptr() for b in blobs], ws.data_ptr(), need, batch, n, 128, 384, 16,
+                                              4, 1e-5, io, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), f"{dtype}"
+    assert L.kfh_single_track_workspace_bytes(1, n, 64, 384, 16, 4) == 0
