@@ -259,6 +259,14 @@ int main(void) {
     if (rc != KFH_EUNSUPPORTED || !strstr(kfh_last_error(), "C=48")) return 4;
     rc = kfh_trimul_forward(0, 0, 0, 0, 0, 0, 0, 1, 8, 128, KFH_OUTGOING, 1e-5f, KFH_BF16, 0);
     if (rc != KFH_EINVAL) return 5;
+    /* a whole block from C: sizes, then the two calls (refused here: null pointers) */
+    if (kfh_pair_block_workspace_bytes(1, 64, 128, 4, 2) == 0) return 6;
+    if (kfh_single_track_workspace_bytes(1, 64, 128, 384, 16, 4) == 0) return 7;
+    rc = kfh_pair_block_forward(0, 0, 0, 0, 0, 0, 0, 0, 0, 1, 64, 128, 4, 2, 1e-5f, KFH_BF16, 0);
+    if (rc != KFH_EINVAL || !strstr(kfh_last_error(), "null")) return 8;
+    rc = kfh_single_track_forward(0, 0, 0, 0, 0, 0, 0, 0, 1, 64, 128, 384, 16, 4, 1e-5f, KFH_BF16, 0);
+    if (rc != KFH_EINVAL || !strstr(kfh_last_error(), "null")) return 9;
+    if (kfh_trimul_row_granule(768, 128) != 256) return 10;
     printf("ok\n");
     return 0;
 }
