@@ -337,8 +337,11 @@ static void work_on(Job* j, Worker* wk) {
     wk->body = j->body;
     wk->kernel = j->name;
     for (;;) {
-        const long long i = j->next.fetch_add(1);
+        long long i = j->next.fetch_add(1);
         if (i >= j->total) break;
+        // schedule 3: the workgroups of a launch in descending order (results may not depend on the
+        // order in which workgroups run: nothing orders them on the GPU)
+        if (g_schedule.load(std::memory_order_relaxed) == 3) i = j->total - 1 - i;
         if (!block_selected(i, j->total)) continue;
         dim3 b((unsigned)(i % j->grid.x), (unsigned)((i / j->grid.x) % j->grid.y),
                (unsigned)(i / ((long long)j->grid.x * j->grid.y)));

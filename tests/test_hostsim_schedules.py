@@ -7,7 +7,8 @@ under three orders — lanes ascending, descending, wavefronts rotating from pas
 give the same bits.  (A race between wavefronts that real hardware would expose shows here as a
 difference; lock-step effects inside one wavefront are outside what the model can vary.)
 
-A fourth run starts every workgroup with all of its LDS overwritten by 0xFF bytes (NaN as bf16 and
+A further run takes the workgroups of every launch in descending order (nothing orders the workgroups
+of a launch on the GPU, so nothing may depend on it), and another starts every workgroup with all of its LDS overwritten by 0xFF bytes (NaN as bf16 and
 fp32): a kernel that reads LDS it has not written itself (left over from the workgroup that ran on
 the compute unit before) gives other bits, or NaN.
 """
@@ -23,7 +24,7 @@ from tests import hostsim
 
 def _run_all(build, run):
     outs = []
-    for mode, poison in ((0, 0), (1, 0), (2, 0), (0, 1)):
+    for mode, poison in ((0, 0), (1, 0), (2, 0), (3, 0), (0, 1)):
         mod = build()
         with torch.no_grad(), hostsim.host_backend():
             hostsim.load().hostsim_set_schedule(mode)
