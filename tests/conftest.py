@@ -12,8 +12,29 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a ROCm GPU (MI355X); run with -m gpu")
 
 
+# GPU tests that have not run on a GPU yet (added after the last GPU run of the suite).  They are
+# collected after the tests that have, so that with `-x` a failure in new code cannot keep tests that
+# were green from running; the allocation-free entry's tests stay last of all.  Move a name out of
+# this set once it has passed on a GPU.
+NOT_YET_RUN_ON_A_GPU = {
+    "test_empty_inputs_give_empty_outputs", "test_pair_block_in_one_c_call", "test_single_track_in_one_c_call",
+    "test_template_batch_at_once_equals_templates_in_turn", "test_template_stack_block_c64",
+    "test_triattn_c64_templates_n384", "test_trimul_c256_tiled_sizes", "test_trimul_other_widths",
+    "test_apb_diffusion_variant_fp32_arithmetic", "test_cross_attention_local_windows_fp32_arithmetic",
+    "test_functional_entry_with_different_query_and_key_tensors", "test_prepared_pair_bias_gives_the_same_bits",
+    "test_caller_workspace_shared_by_consecutive_ops", "test_phases_over_row_ranges_at_the_benchmark_size",
+    "test_phases_over_row_ranges_give_the_same_bits", "test_gpu_results_against_the_host_builds",
+}
+
+
 def pytest_collection_modifyitems(config, items):
     import torch
+
+    def rank(item):
+        if item.nodeid.startswith("tests/test_zz_no_alloc.py"):
+            return 2
+        return 1 if "gpu" in item.keywords and item.originalname in NOT_YET_RUN_ON_A_GPU else 0
+    items.sort(key=rank)              # stable: the order inside each group stays as collected
 
     if torch.cuda.is_available():
         return

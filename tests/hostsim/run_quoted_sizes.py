@@ -13,7 +13,7 @@ from __future__ import annotations
 import sys
 import time
 
-import tests.test_block_gpu as BK
+import tests.test_zx_row_ranges_gpu as BK
 import tests.test_quoted_sizes_gpu as Q
 import tests.test_shipping_dims_gpu as SD
 import tests.test_triattn_gpu as TA

@@ -30,6 +30,7 @@ GPU_MODULES = [
     "tests.test_block_gpu",
     "tests.test_shipping_dims_gpu",
     "tests.test_parcae_gpu",
+    "tests.test_zx_row_ranges_gpu",
     "tests.test_zy_host_model_vectors_gpu",
     "tests.test_zz_no_alloc",
 ]
