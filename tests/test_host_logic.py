@@ -413,3 +413,68 @@ def test_block_with_phases_over_row_ranges(rec):
         blk(small, torch.ones(1, 70, 70, dtype=torch.bool), inplace_output=True)
     assert rec.names(("_forward",)) == ["kfh_trimul_forward", "kfh_trimul_forward", "kfh_triattn_forward",
                                         "kfh_triattn_forward", "kfh_transition_forward"]
+
+
+def test_phased_op_on_two_streams_orders_core_and_output(rec, monkeypatch):
+    """The two-stream form of an op run in row ranges, with stand-ins for the streams and events: the
+    input phase and every core phase are enqueued on the caller's stream, each output phase on the side
+    stream after an event recorded behind its core phase, and the caller's stream waits for the side
+    stream at the end."""
+    from kfold_amd import _lib, ops
+
+    log = []
+
+    class FakeStream:
+        def __init__(self, name):
+            self.name, self.cuda_stream = name, 0
+
+        def wait_event(self, ev):
+            log.append((self.name, "wait_event", ev.id))
+
+        def wait_stream(self, other):
+            log.append((self.name, "wait_stream", other.name))
+
+    class FakeEvent:
+        count = 0
+
+        def __init__(self):
+            FakeEvent.count += 1
+            self.id = FakeEvent.count
+
+        def record(self, stream):
+            log.append((stream.name, "record", self.id))
+
+    main, side = FakeStream("main"), FakeStream("side")
+    current = [main]
+
+    class use_stream:
+        def __init__(self, s):
+            self.s = s
+
+        def __enter__(self):
+            self.prev, current[0] = current[0], self.s
+
+        def __exit__(self, *a):
+            current[0] = self.prev
+
+    monkeypatch.setattr(torch.cuda, "current_stream", lambda dev=None: current[0])
+    monkeypatch.setattr(torch.cuda, "Event", FakeEvent)
+    monkeypatch.setattr(torch.cuda, "stream", use_stream)
+    monkeypatch.setattr(ops, "_stream", lambda dev: log.append((current[0].name, "launch")) or 0)
+
+    N = 300
+    z = torch.zeros(1, N, N, 128, dtype=torch.bfloat16)
+    blob = torch.zeros(_lib.lib().kfh_trimul_packed_bytes(128), dtype=torch.uint8)
+    waits = []
+    ops.trimul_forward(z, torch.ones(1, N, N, dtype=torch.bool), blob, "outgoing", residual=z, out=z,
+                       row_chunks=3, side=side, before_write=lambda: waits.append(len(log)))
+    IN, CORE, OUT = _lib.KFH_STAGE_IN, _lib.KFH_STAGE_CORE, _lib.KFH_STAGE_OUT
+    calls = [(c[13], c[14], c[15]) for c in rec.of("kfh_trimul_forward_rows")]
+    assert calls == [(IN, 0, N), (CORE, 0, 128), (OUT, 0, 128), (CORE, 128, 128), (OUT, 128, 128),
+                     (CORE, 256, 44), (OUT, 256, 44)]
+    assert log == [("main", "launch"),                                             # input phase
+                   ("main", "launch"), ("main", "record", 1), ("side", "wait_event", 1), ("side", "launch"),
+                   ("main", "launch"), ("main", "record", 2), ("side", "wait_event", 2), ("side", "launch"),
+                   ("main", "launch"), ("main", "record", 3), ("side", "wait_event", 3), ("side", "launch"),
+                   ("main", "wait_stream", "side")]
+    assert waits == [1], "the caller's wait comes right after the input phase, before anything is written"
