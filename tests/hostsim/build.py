@@ -24,15 +24,11 @@ OBJ = HERE / "_obj"
 CXX = os.environ.get("HOSTSIM_CXX", "/opt/rocm/llvm/bin/clang++")
 FLAGS = ["-x", "c++", "-std=c++17", "-O2", "-march=x86-64-v3", "-fPIC", "-pthread", "-w",
          f"-I{HERE}", "-ffp-contract=off"]
-# extra compiler flags for a checking build, e.g.
-#   HOSTSIM_EXTRA_FLAGS="-fsanitize=alignment -fsanitize-trap=alignment" python tests/hostsim/build.py -f
-# makes every load and store through a typed pointer (the 16-byte fragment loads, the packed 4- and
-# 8-byte stores) trap unless the address has the type's alignment;
-#   HOSTSIM_EXTRA_FLAGS="-g -fsanitize=signed-integer-overflow,unsigned-integer-overflow,implicit-signed-integer-truncation,implicit-unsigned-integer-truncation,shift
-#                        -fsanitize-trap=all -fsanitize-ignorelist=tests/hostsim/ubsan_ignore.txt"
-# traps on index arithmetic that overflows or is cut to 32 bits (hostsim.cpp reports the kernel,
-# workgroup, thread and library offset of a trap; `llvm-symbolizer -e libkfold_hostsim.so -i OFFSET`
-# names the source line)
+# HOSTSIM_EXTRA_FLAGS: extra host-compiler flags for a checking build of this library: clang's
+# undefined-behaviour checks in trapping mode (alignment of every typed load and store; signed and
+# unsigned overflow and 64 -> 32 bit truncation of index arithmetic, with ubsan_ignore.txt listing
+# the one intended wrap; bounds of the per-lane arrays).  hostsim.cpp reports the kernel, workgroup,
+# thread and library offset of a trap; the README lists the command lines.
 FLAGS += os.environ.get("HOSTSIM_EXTRA_FLAGS", "").split()
 
 

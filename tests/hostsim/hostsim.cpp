@@ -499,7 +499,7 @@ static void segv_handler(int sig, siginfo_t* info, void*) {
     sigaction(sig, sig == SIGSEGV ? &g_old_segv : &g_old_bus, nullptr);
 }
 
-// A trap of a checking build (HOSTSIM_EXTRA_FLAGS with -fsanitize-trap): say where, as an offset
+// A trap of a checking build (HOSTSIM_EXTRA_FLAGS with the compiler's checks in trapping mode): say where, as an offset
 // into this library that `llvm-symbolizer -e libkfold_hostsim.so` resolves when built with -g.
 static struct sigaction g_old_ill;
 static void ill_handler(int sig, siginfo_t* info, void*) {
